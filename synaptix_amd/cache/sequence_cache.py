@@ -5,7 +5,8 @@ Layers with the same needs (kv heads, head size, all keys or a window of them) f
 group has storage and a page pool of its own:
     k_pages [layers, pages, kv_heads, 64, head_dim]
     v_pages [layers, pages, kv_heads, head_dim, 64]      (transposed inside the page; a bf16 page in the
-                                                          order of its kernels, ops.v_pages_to_kernel_order)
+                                                          order of its kernels, ops.v_pages_to_kernel_order;
+                                                          KvNeed.v_heads of them where kv heads share values)
 A group that keeps a window gives pages back as soon as every position in them has left the
 window.  Layers with a StateNeed get `state[layer] : [slots + 1, *shape]`, zeroed when a slot is
 taken (the reference keeps such state in the same per-layer vector as the keys and values,
@@ -142,7 +143,7 @@ class SequenceCache:
             # zeros: what a kernel may touch beyond a sequence's end is at least a number
             g.spare_page = g.n_pages
             g.k = torch.zeros((n, g.n_pages + 1, nd.kv_heads, PAGE_TOKENS, nd.head_dim), dtype=dtype, device=self.device)
-            g.v = torch.zeros((n, g.n_pages + 1, nd.kv_heads, nd.v_dim or nd.head_dim, PAGE_TOKENS), dtype=dtype,
+            g.v = torch.zeros((n, g.n_pages + 1, nd.v_heads or nd.kv_heads, nd.v_dim or nd.head_dim, PAGE_TOKENS), dtype=dtype,
                               device=self.device)
 
     def _register(self, key, need) -> None:
@@ -302,5 +303,6 @@ class SequenceCache:
 
     def bytes_per_token(self) -> int:
         el = torch.empty(0, dtype=self.dtype).element_size()
-        return sum(len(g.layers) * g.need.kv_heads * (g.need.head_dim + (g.need.v_dim or g.need.head_dim)) * el
+        return sum(len(g.layers) * (g.need.kv_heads * g.need.head_dim
+                                    + (g.need.v_heads or g.need.kv_heads) * (g.need.v_dim or g.need.head_dim)) * el
                    for g in self.groups)

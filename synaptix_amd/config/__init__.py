@@ -2,8 +2,9 @@ from .errors import ConfigError
 from .qwen3 import Qwen3Config
 from .bizipel import BizipelConfig
 from .kamivik import KamivikConfig
+from .repolix import RepolixConfig
 from .registry import (Architecture, register_architecture, resolve_architecture, known_architectures,
                        load_config, read_config_json)
 
-__all__ = ["ConfigError", "Qwen3Config", "BizipelConfig", "KamivikConfig", "Architecture", "register_architecture", "resolve_architecture",
+__all__ = ["ConfigError", "Qwen3Config", "BizipelConfig", "KamivikConfig", "RepolixConfig", "Architecture", "register_architecture", "resolve_architecture",
            "known_architectures", "load_config", "read_config_json"]

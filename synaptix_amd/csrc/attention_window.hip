@@ -6,6 +6,8 @@
 //   p_j = exp(score_j) / (sink + sum_j exp(score_j)),  sink = 1 with `sink_one` (a further key of score 0 that has
 //       no value), else 0;
 //   head h reads kv head h / (heads / kv heads); keys have `dim` values, values `vdim`;
+//   v_share > 1: that many neighbouring kv heads read the values of one value head (kv heads / v_share of them are
+//       stored), as the maps of a differential attention do, which have keys of their own and the values in common;
 //   the heads' results may be multiplied by sigmoid(gate) before they are stored.
 // Scores, weights and sums are 32-bit whatever the cache's type; the weights are not rounded before they meet V.
 //
@@ -24,22 +26,27 @@ struct WindowTerms {
   int window;            // 0: every key
   int keep_first;
   int sink_one;
+  int v_share;           // this many neighbouring kv heads read one value head (1: each its own)
 };
 
 // ---------------------------------------------------------------- intake: bias, q/k norm, cache write
 // proj [N][width] float holds the fused projection  [q heads x dim | k heads x dim | v heads x vdim | ...]; what lies
-// behind v (a gate) is left where it is.  One wave for each (token, q head | k head | v head).
+// behind v (a gate) is left where it is.  One wave for each (token, q head | k head | v head); there are nv value
+// heads (nkv, unless several kv heads share a value head).
+// cos_t, sin_t [positions][rot / 2] (or null): after the norm the first `rot` values of a q or k head are turned, value
+// i < rot / 2 paired with value i + rot / 2, by the angle whose cosine and sine stand at [position][i].
 template <typename T>
 __global__ void window_intake_kernel(const float* __restrict__ proj, int width, const float* __restrict__ bias,
                                      T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
                                      const int* __restrict__ page_table, int table_stride,
                                      const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                      const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
-                                     int nh, int nkv, int dim, int vdim, int write_kv) {
+                                     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
+                                     int nh, int nkv, int nv, int dim, int vdim, int write_kv) {
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
   const int tok = blockIdx.x;
   const int item = blockIdx.y * (blockDim.x / SYN_WAVE) + wave;
-  if (item >= (write_kv ? nh + 2 * nkv : nh)) return;
+  if (item >= (write_kv ? nh + nkv + nv : nh)) return;
   const bool is_q = item < nh, is_k = !is_q && item < nh + nkv;
   const int len = (is_q || is_k) ? dim : vdim;
   const int col = is_q ? item * dim : (is_k ? nh * dim + (item - nh) * dim : (nh + nkv) * dim + (item - nh - nkv) * vdim);
@@ -65,36 +72,47 @@ __global__ void window_intake_kernel(const float* __restrict__ proj, int width, 
     if (is_k) {
       dst = k_pages + (((size_t)page * nkv + (item - nh)) * SYN_PAGE + pos % SYN_PAGE) * dim;
     } else {
-      dst = v_pages + ((size_t)page * nkv + (item - nh - nkv)) * vdim * SYN_PAGE + pos % SYN_PAGE;
+      dst = v_pages + ((size_t)page * nv + (item - nh - nkv)) * vdim * SYN_PAGE + pos % SYN_PAGE;
       stride = SYN_PAGE;
     }
   }
+  const int half = (cos_t && (is_q || is_k)) ? rot / 2 : 0;
   for (int d = lane; d < len; d += SYN_WAVE) {
     float v = src[d] + (b ? b[d] : 0.f);
     if (gain) v = v * inv * gain[d];
+    if (d < 2 * half) {
+      const int i = d < half ? d : d - half, mate = d < half ? d + half : d - half;
+      float o = src[mate] + (b ? b[mate] : 0.f);
+      if (gain) o = o * inv * gain[mate];
+      const float c = cos_t[(size_t)pos * half + i], sn = sin_t[(size_t)pos * half + i];
+      v = d < half ? v * c - o * sn : v * c + o * sn;
+    }
     dst[(size_t)d * stride] = from_f32<T>(v);
   }
 }
 
 SYN_EXPORT int syn_window_intake(const float* proj, int width, const float* bias, void* q_out, void* k_pages,
                                  void* v_pages, int is_f32, const int* page_table, int table_stride, const int* tok_seq,
-                                 const int* tok_pos, const float* q_gain, const float* k_gain, float eps, int n_tokens,
-                                 int nh, int nkv, int dim, int vdim, int write_kv, hipStream_t stream) {
-  SYN_CHECK(n_tokens > 0 && nh > 0 && nkv > 0 && dim > 0 && vdim > 0, "window_intake: empty input");
-  SYN_CHECK(width >= (nh + nkv) * dim + nkv * vdim, "window_intake: rows of %d values do not hold q, k and v", width);
+                                 const int* tok_pos, const float* q_gain, const float* k_gain, float eps,
+                                 const float* cos_t, const float* sin_t, int rot, int n_tokens,
+                                 int nh, int nkv, int nv, int dim, int vdim, int write_kv, hipStream_t stream) {
+  SYN_CHECK(n_tokens > 0 && nh > 0 && nkv > 0 && nv > 0 && dim > 0 && vdim > 0, "window_intake: empty input");
+  SYN_CHECK(width >= (nh + nkv) * dim + nv * vdim, "window_intake: rows of %d values do not hold q, k and v", width);
   SYN_CHECK((q_gain == nullptr) == (k_gain == nullptr), "window_intake: q and k gains come together");
-  const int wpb = 4, items = write_kv ? nh + 2 * nkv : nh;
+  SYN_CHECK((cos_t == nullptr) == (sin_t == nullptr) && (cos_t == nullptr || (rot > 0 && rot % 2 == 0 && rot <= dim)),
+            "window_intake: a rotation of %d of %d values", rot, dim);
+  const int wpb = 4, items = write_kv ? nh + nkv + nv : nh;
   const dim3 grid(n_tokens, (items + wpb - 1) / wpb);
   if (is_f32)
     window_intake_kernel<float><<<grid, wpb * SYN_WAVE, 0, stream>>>(proj, width, bias, (float*)q_out, (float*)k_pages,
                                                                      (float*)v_pages, page_table, table_stride, tok_seq,
-                                                                     tok_pos, q_gain, k_gain, eps, nh, nkv, dim, vdim,
-                                                                     write_kv);
+                                                                     tok_pos, q_gain, k_gain, eps, cos_t, sin_t, rot, nh,
+                                                                     nkv, nv, dim, vdim, write_kv);
   else
     window_intake_kernel<bf16><<<grid, wpb * SYN_WAVE, 0, stream>>>(proj, width, bias, (bf16*)q_out, (bf16*)k_pages,
                                                                     (bf16*)v_pages, page_table, table_stride, tok_seq,
-                                                                    tok_pos, q_gain, k_gain, eps, nh, nkv, dim, vdim,
-                                                                    write_kv);
+                                                                    tok_pos, q_gain, k_gain, eps, cos_t, sin_t, rot, nh,
+                                                                    nkv, nv, dim, vdim, write_kv);
   SYN_LAUNCH_CHECK("window_intake");
   return 0;
 }
@@ -160,7 +178,7 @@ window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, 
     const int kb = idx < n_kept_blocks ? idx : first_window_block + (idx - n_kept_blocks);
     const int page = page_table[(size_t)seq * table_stride + kb];
     const size_t kbase = ((size_t)page * nkv + kvh) * SYN_PAGE * dim;
-    const size_t vbase = ((size_t)page * nkv + kvh) * SYN_PAGE * vdim;
+    const size_t vbase = ((size_t)page * (nkv / terms.v_share) + kvh / terms.v_share) * SYN_PAGE * vdim;
     const int key = kb * SYN_PAGE + lane;
     const bool valid = key <= pos && (key >= lo || key < kept);
     float s = -INFINITY;
@@ -254,8 +272,9 @@ SYN_EXPORT int syn_window_attention(const void* q, const void* k_pages, const vo
                                     const float* gate, int gate_stride, const float* gate_bias, void* out, float scale,
                                     int n_tokens, int nh, int nkv, int dim, int vdim, const float* slopes,
                                     const float* r1, const float* r2, float softcap, int window, int keep_first,
-                                    int sink_one, hipStream_t stream) {
+                                    int sink_one, int v_share, hipStream_t stream) {
   SYN_CHECK(n_tokens > 0 && nh > 0 && nkv > 0, "window_attention: empty input");
+  SYN_CHECK(v_share > 0 && nkv % v_share == 0, "window_attention: %d kv heads in shares of %d", nkv, v_share);
   SYN_CHECK(nh % nkv == 0, "window_attention: %d heads do not divide into %d kv heads", nh, nkv);
   SYN_CHECK(dim > 0 && dim <= AW_MAX_DIM && vdim > 0 && vdim <= AW_MAX_DIM,
             "window_attention: head sizes %d and %d are outside 1..%d", dim, vdim, AW_MAX_DIM);
@@ -263,7 +282,7 @@ SYN_EXPORT int syn_window_attention(const void* q, const void* k_pages, const vo
             (double)softcap, window, keep_first);
   SYN_CHECK((r1 == nullptr) == (r2 == nullptr), "window_attention: r1 and r2 come together");
   SYN_CHECK(gate == nullptr || gate_stride >= nh * vdim, "window_attention: gate rows of %d values", gate_stride);
-  const WindowTerms terms = {slopes, r1, r2, softcap, window, keep_first, sink_one};
+  const WindowTerms terms = {slopes, r1, r2, softcap, window, keep_first, sink_one, v_share};
   const dim3 grid(n_tokens, nh);
   // few (token, head) pairs (single tokens of a few sequences): eight waves share each pair's keys
   const bool many_waves = (long)n_tokens * nh < 8L * syn_compute_units();
@@ -387,7 +406,7 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
   auto fetch = [&](int idx) {
     const int page = page_table[(size_t)seq * table_stride + block_of(idx)];
     const uint4* kp = (const uint4*)(k_pages + ((size_t)page * nkv + kvh) * SYN_PAGE * dim);
-    const uint4* vp = (const uint4*)(v_pages + ((size_t)page * nkv + kvh) * SYN_PAGE * vdim);
+    const uint4* vp = (const uint4*)(v_pages + ((size_t)page * (nkv / terms.v_share) + kvh / terms.v_share) * SYN_PAGE * vdim);
 #pragma unroll
     for (int r = 0; r < PIECES; ++r) {
       const int it = tid + 256 * r;
@@ -526,8 +545,9 @@ SYN_EXPORT int syn_window_attention_prefill_bf16(const void* q, const void* k_pa
                                                  int gate_stride, const float* gate_bias, void* out, float scale, int nh,
                                                  int nkv, int dim, int vdim, const float* slopes, const float* r1,
                                                  const float* r2, float softcap, int window, int keep_first, int sink_one,
-                                                 hipStream_t stream) {
+                                                 int v_share, hipStream_t stream) {
   SYN_CHECK(n_tokens > 0 && n_seqs > 0 && nh > 0 && nkv > 0, "window_attention_prefill: empty input");
+  SYN_CHECK(v_share > 0 && nkv % v_share == 0, "window_attention_prefill: %d kv heads in shares of %d", nkv, v_share);
   SYN_CHECK(nh % nkv == 0, "window_attention_prefill: %d heads do not divide into %d kv heads", nh, nkv);
   SYN_CHECK(dim % 16 == 0 && vdim % 16 == 0 && dim >= 16 && vdim >= 16 && dim <= 16 * AWP_TILES && vdim <= 16 * AWP_TILES,
             "window_attention_prefill: head sizes %d and %d (multiples of 16 up to %d)", dim, vdim, 16 * AWP_TILES);
@@ -538,7 +558,7 @@ SYN_EXPORT int syn_window_attention_prefill_bf16(const void* q, const void* k_pa
             "window_attention_prefill: gate rows of %d values", gate_stride);
   SYN_CHECK((uintptr_t)q % 16 == 0 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0 && (uintptr_t)out % 8 == 0,
             "window_attention_prefill: operands are not aligned");
-  const WindowTerms terms = {slopes, r1, r2, softcap, window, keep_first, sink_one};
+  const WindowTerms terms = {slopes, r1, r2, softcap, window, keep_first, sink_one, v_share};
   const dim3 grid((n_tokens + 63) / 64 + n_seqs, nh);      // at most this many tiles of 64 queries; the rest leave at once
   if (dim % 32 == 0)
     window_prefill_bf16_kernel<true><<<grid, 256, 0, stream>>>(

@@ -110,7 +110,8 @@ __device__ __forceinline__ float load_gain(const void* w, int is_f32, int i, flo
 // another activation is another case here and another name in the host's table.
 #define SYN_ACT_SILU 0
 #define SYN_ACT_GELU_TANH 1
-#define SYN_ACT_COUNT 2
+#define SYN_ACT_SWIGLU_LIMIT 2   // both inputs bounded by a limit, a steeper sigmoid, and one added to the linear half
+#define SYN_ACT_COUNT 3
 __device__ __forceinline__ float gate_activation(int act, float g) {
   switch (act) {
     case SYN_ACT_GELU_TANH:  // 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))
@@ -119,7 +120,15 @@ __device__ __forceinline__ float gate_activation(int act, float g) {
       return g / (1.f + expf(-g));
   }
 }
-__device__ __forceinline__ float gated(int act, float gate, float up) { return gate_activation(act, gate) * up; }
+// limit: the bound of SYN_ACT_SWIGLU_LIMIT (g <- min(g, limit), u <- clamp(u, -limit, limit);
+// g sigmoid(1.702 g) (u + 1)); the other activations do not read it
+__device__ __forceinline__ float gated(int act, float gate, float up, float limit = 0.f) {
+  if (act == SYN_ACT_SWIGLU_LIMIT) {
+    const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
+    return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+  }
+  return gate_activation(act, gate) * up;
+}
 
 // ---- what an attention kernel may do to a scaled score before the mask and the softmax ----
 // A soft cap, cap * tanh(score / cap), and a penalty in the distance between query and key, - slope[head] * (q - k)

@@ -12,42 +12,42 @@
 SYN_DEFINE_ERROR_CHANNEL
 
 // ------------------------------------------------------------------ embedding
-// resid[n, :] = table[ids[n], :] widened to float.  Ids are checked on the host.
+// resid[n, :] = scale * table[ids[n], :] widened to float.  Ids are checked on the host.
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids, float* __restrict__ resid,
-                             int H) {
+                             int H, float scale) {
   const int n = blockIdx.x;
   const T* row = table + (size_t)ids[n] * H;
   float* out = resid + (size_t)n * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_f32<T>(row[i]);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_f32<T>(row[i]) * scale;
 }
 
 // the same from a bf16 table in fragment order ([V / 16][H / 32][64 lanes][8], as the products read the tied
 // output head): eight consecutive values of a row are one lane's 16 bytes
 __global__ void embed_packed_kernel(const bf16* __restrict__ table, const int* __restrict__ ids, float* __restrict__ resid,
-                                    int H) {
+                                    int H, float scale) {
   const int n = blockIdx.x, id = ids[n];
   const bf16* group = table + (size_t)(id / 16) * H * 16;   // the 16 rows around row id: H / 32 fragments of 512 values
   float* out = resid + (size_t)n * H;
   for (int c = threadIdx.x; c < H / 8; c += blockDim.x) {   // chunk c: values 8 c .. 8 c + 7 of the row
     const bf16x8 v = *(const bf16x8*)(group + (size_t)(c / 4) * 512 + ((c % 4) * 16 + id % 16) * 8);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) out[c * 8 + e] = (float)v[e];
+    for (int e = 0; e < 8; ++e) out[c * 8 + e] = (float)v[e] * scale;
   }
 }
 
 // table_kind: 0 = bf16 rows, 1 = float rows, 2 = bf16 in fragment order (V a multiple of 16, H of 32)
 SYN_EXPORT int syn_embed(const void* table, int table_kind, const int* ids, float* resid, int n_tokens, int H,
-                         hipStream_t stream) {
+                         float scale, hipStream_t stream) {
   SYN_CHECK(n_tokens > 0 && H > 0, "embed: empty input (%d tokens, width %d)", n_tokens, H);
   SYN_CHECK(table_kind >= 0 && table_kind <= 2, "embed: unknown kind of table %d", table_kind);
   if (table_kind == 1) {
-    embed_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)table, ids, resid, H);
+    embed_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)table, ids, resid, H, scale);
   } else if (table_kind == 2) {
     SYN_CHECK(H % 32 == 0, "embed: a table in fragment order has a width that is a multiple of 32, not %d", H);
-    embed_packed_kernel<<<n_tokens, 256, 0, stream>>>((const bf16*)table, ids, resid, H);
+    embed_packed_kernel<<<n_tokens, 256, 0, stream>>>((const bf16*)table, ids, resid, H, scale);
   } else {
-    embed_kernel<bf16><<<n_tokens, 256, 0, stream>>>((const bf16*)table, ids, resid, H);
+    embed_kernel<bf16><<<n_tokens, 256, 0, stream>>>((const bf16*)table, ids, resid, H, scale);
   }
   SYN_LAUNCH_CHECK("embed");
   return 0;
@@ -234,19 +234,20 @@ SYN_EXPORT int syn_rmsnorm_rows(const void* x, int is_f32, const void* gain, int
 // ------------------------------------------------------------------ SwiGLU on a fused [gate | up] row
 // out[n, i] = act(gu[n, i]) * gu[n, I + i] in 32-bit (gate_activation; silu(z) = z / (1 + exp(-z))).
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_rows, int I, int act) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_rows, int I, int act, float limit) {
   const size_t total = (size_t)n_rows * I;
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
     const size_t n = idx / I;
     const int i = (int)(idx - n * I);
     const float g = to_f32<T>(gu[n * 2 * I + i]);
     const float u = to_f32<T>(gu[n * 2 * I + I + i]);
-    out[idx] = from_f32<T>(gated(act, g, u));
+    out[idx] = from_f32<T>(gated(act, g, u, limit));
   }
 }
 
 // 8 values a thread with 16-byte loads (bf16, width a multiple of 8)
-__global__ void swiglu_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int n_rows, int I, int act) {
+__global__ void swiglu_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int n_rows, int I, int act,
+                                   float limit) {
   const int I8 = I / 8;
   const size_t total = (size_t)n_rows * I8;
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
@@ -256,19 +257,20 @@ __global__ void swiglu_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict
     const bf16x8 u = *(const bf16x8*)(gu + n * 2 * I + I + i);
     bf16x8 o;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) o[e] = (bf16)gated(act, (float)g[e], (float)u[e]);
+    for (int e = 0; e < 8; ++e) o[e] = (bf16)gated(act, (float)g[e], (float)u[e], limit);
     *(bf16x8*)(out + n * I + i) = o;
   }
 }
 
-SYN_EXPORT int syn_swiglu(const void* gu, void* out, int is_f32, int n_rows, int I, int act, hipStream_t stream) {
+SYN_EXPORT int syn_swiglu(const void* gu, void* out, int is_f32, int n_rows, int I, int act, float limit,
+                          hipStream_t stream) {
   SYN_CHECK(n_rows > 0 && I > 0, "swiglu: empty input (%d rows, width %d)", n_rows, I);
   SYN_CHECK(act >= 0 && act < SYN_ACT_COUNT, "swiglu: unknown activation code %d", act);
   if (!is_f32 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
     const size_t total = (size_t)n_rows * (I / 8);
     int grid = (int)((total + 255) / 256);
     if (grid > 65536) grid = 65536;
-    swiglu_vec8_kernel<<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, n_rows, I, act);
+    swiglu_vec8_kernel<<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, n_rows, I, act, limit);
     SYN_LAUNCH_CHECK("swiglu");
     return 0;
   }
@@ -276,9 +278,9 @@ SYN_EXPORT int syn_swiglu(const void* gu, void* out, int is_f32, int n_rows, int
   int grid = (int)((total + 255) / 256);
   if (grid > 65536) grid = 65536;
   if (is_f32)
-    swiglu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu, (float*)out, n_rows, I, act);
+    swiglu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu, (float*)out, n_rows, I, act, limit);
   else
-    swiglu_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, n_rows, I, act);
+    swiglu_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, n_rows, I, act, limit);
   SYN_LAUNCH_CHECK("swiglu");
   return 0;
 }

@@ -30,6 +30,7 @@
 struct Epilogue {
   int out_is_f32;
   int act;
+  float limit;      // the bound of an activation that has one (gated, csrc/common.h)
 };
 
 // ------------------------------------------------------------------ SIMT, any type
@@ -143,7 +144,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
       const int m = 4 * (ln / 16) + j, col = (int)blockIdx.x * 16 + ln % 16;  // N / 2 outputs, 16 a workgroup
       if (m < M && 2 * col < N) {
         const float g = summed(0, j, ln), up = summed(1, j, ln);
-        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, g, up);
+        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, g, up, ep.limit);
       }
     }
   } else {
@@ -311,7 +312,7 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
       if (m < M && 2 * col < N) {
         const float f = rn.ss ? inv[m] : 1.f;
         const float g = summed(0, j, ln) * f, up = summed(1, j, ln) * f;
-        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, g, up);
+        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, g, up, ep.limit);
       }
     }
   } else {
@@ -396,7 +397,7 @@ gemm_packed2_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, voi
       const int m = 4 * (ln / 16) + j, col = (int)blockIdx.x * 16 + ln % 16;  // N / 2 outputs, 16 a workgroup
       if (m < M && 2 * col < N) {
         const float f = rn.ss ? inv[m] : 1.f;
-        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, summed(0, j, ln) * f, summed(1, j, ln) * f);
+        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, summed(0, j, ln) * f, summed(1, j, ln) * f, ep.limit);
       }
     }
   } else {
@@ -469,10 +470,10 @@ __device__ __forceinline__ void store_tiles(const f32x16 (&acc)[TM][TN], void* _
             const float own1 = acc[i][j + 1 < TN ? j + 1 : j][e], other1 = __shfl_xor(own1, 16, SYN_WAVE);
             const float g = first ? own0 : other1, up = first ? other0 : own1;
             if (m < M && nw + (j + (first ? 0 : 1)) * 32 < N)
-              ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 32] = (bf16)gated(ep.act, g, up);
+              ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 32] = (bf16)gated(ep.act, g, up, ep.limit);
           } else {
             if (m < M && nw + j * 32 < N && first)
-              ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 16] = (bf16)gated(ep.act, own0, other0);
+              ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 16] = (bf16)gated(ep.act, own0, other0, ep.limit);
           }
         }
   } else {
@@ -1046,7 +1047,7 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
     return 0;
   }
   const int out_is_f32 = dtype == 2;
-  const Epilogue ep = {out_is_f32, SYN_ACT_SILU};   // (no activation in a plain product)
+  const Epilogue ep = {out_is_f32, SYN_ACT_SILU, 0.f};   // (no activation in a plain product)
   const bool aligned = (K % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
   SYN_CHECK(slices == 1 || aligned, "gemm: slices of K need 16-byte aligned operands");
   if (force_simt || !aligned) {
@@ -1116,12 +1117,12 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
 // turns of 16: rows 32b .. 32b+15 are rows 16b .. 16b+15 of Wg, rows 32b+16 .. 32b+31 those of Wu.
 // The activation is applied to the 32-bit sums and rounded once.
 // w_packed: as for syn_gemm
-SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, int N, int K, int act, int w_packed,
-                               hipStream_t stream) {
+SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, int N, int K, int act, float limit,
+                               int w_packed, hipStream_t stream) {
   SYN_CHECK(M > 0 && N > 0 && K > 0, "gemm_swiglu: empty shape M=%d N=%d K=%d", M, N, K);
   SYN_CHECK(!w_packed || K % 128 == 0, "gemm_swiglu: a weight in fragment order needs K = %d a multiple of 128", K);
   SYN_CHECK(act >= 0 && act < SYN_ACT_COUNT, "gemm_swiglu: unknown activation code %d", act);
-  const Epilogue ep = {0, act};
+  const Epilogue ep = {0, act, limit};
   SYN_CHECK(N % 32 == 0, "gemm_swiglu: %d paired rows are no multiple of 32", N);
   SYN_CHECK(K % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0,
             "gemm_swiglu: K = %d must be a multiple of 8 and the operands 16-byte aligned", K);
@@ -1165,13 +1166,13 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
 //   resid [M, N] float (or null; then float sums, one slice, not paired, `out` unused): resid += sums,
 //   xs [M, N] bf16 = (gain_offset + gain[n]) * resid, ss_out [M, N / 16] = sums of resid^2 over groups of 16 columns.
 SYN_EXPORT int syn_gemm_packed_norm(const void* x, const void* wp, void* out, int out_code, int M, int N, int K, int paired,
-                                    int act, int slices, const float* ss, int ss_groups, int norm_dim, float eps,
+                                    int act, float limit, int slices, const float* ss, int ss_groups, int norm_dim, float eps,
                                     float* resid, void* xs, float* ss_out, const void* gain, int gain_is_f32,
                                     float gain_offset, hipStream_t stream) {
   SYN_CHECK(act >= 0 && act < SYN_ACT_COUNT, "gemm_packed: unknown activation code %d", act);
   SYN_CHECK(slices >= 1 && slices <= 64 && (slices == 1 || (out_code == 2 && !paired)),
             "gemm_packed: %d slices of K need a float output [slices, M, N] and no activation", slices);
-  const Epilogue ep = {out_code == 2, act};
+  const Epilogue ep = {out_code == 2, act, limit};
   SYN_CHECK(M > 0 && M <= 16 && N > 0 && K > 0, "gemm_packed: M = %d (1 .. 16), N = %d, K = %d", M, N, K);
   SYN_CHECK(N % 16 == 0 && K % 32 == 0 && (!paired || N % 32 == 0),
             "gemm_packed: N = %d must be a multiple of 16 (32 for paired rows), K = %d of 32", N, K);
@@ -1209,7 +1210,7 @@ SYN_EXPORT int syn_gemm_packed_norm(const void* x, const void* wp, void* out, in
 }
 
 SYN_EXPORT int syn_gemm_packed(const void* x, const void* wp, void* out, int out_code, int M, int N, int K, int paired,
-                               int act, int slices, hipStream_t stream) {
-  return syn_gemm_packed_norm(x, wp, out, out_code, M, N, K, paired, act, slices, nullptr, 0, 0, 0.f, nullptr, nullptr,
+                               int act, float limit, int slices, hipStream_t stream) {
+  return syn_gemm_packed_norm(x, wp, out, out_code, M, N, K, paired, act, limit, slices, nullptr, 0, 0, 0.f, nullptr, nullptr,
                               nullptr, nullptr, 0, 0.f, stream);
 }

@@ -441,6 +441,138 @@ SYN_EXPORT int syn_route_topk(const float* logits, const float* bias, int* ids, 
   return 0;
 }
 
+// ---------------------------------------------------------------- a router that scores all experts
+// s = softmax(logits) over all E outputs (32-bit).  The choice is made on s + correction: the E outputs form n_groups
+// equal groups of neighbours, a group's score is its largest choice score, only members of the keep_groups best groups
+// can be chosen (the others count as minus infinity), and of those the `top` largest are taken (the lower index of
+// equal ones, for groups and for experts).  weights: the chosen experts' s itself, without the correction; renorm:
+// divided by their sum.  One wave a token.
+__global__ void __launch_bounds__(256) route_scores_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
+                                                           int* __restrict__ ids, float* __restrict__ weights, int n_tokens,
+                                                           int E, int top, int n_groups, int keep_groups, int renorm) {
+  __shared__ float ss[4][ROUTE_MAX_EXPERTS];       // the scores
+  __shared__ float cs[4][ROUTE_MAX_EXPERTS];       // the choice scores
+  __shared__ float gs[4][ROUTE_MAX_EXPERTS];       // the groups' scores
+  __shared__ float chosen_s[4][ROUTE_MAX_TOP];
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE, tok = blockIdx.x * 4 + wave;
+  if (tok >= n_tokens) return;             // (waves work alone: no barrier of the workgroup below)
+  float* sc = ss[wave];
+  float* c = cs[wave];
+  float* grp = gs[wave];
+  float* chosen = chosen_s[wave];
+  auto wave_sync = [] {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  float mx = -INFINITY;
+  for (int e = lane; e < E; e += SYN_WAVE) mx = fmaxf(mx, logits[(size_t)tok * E + e]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += SYN_WAVE) {
+    const float p = expf(logits[(size_t)tok * E + e] - mx);
+    sc[e] = p;
+    sum += p;
+  }
+  sum = wave_sum(sum);
+  const int per = E / n_groups;
+  for (int e = lane; e < E; e += SYN_WAVE) {
+    sc[e] = sc[e] / sum;
+    c[e] = sc[e] + (correction ? correction[e] : 0.f);
+  }
+  wave_sync();
+  if (keep_groups < n_groups) {
+    for (int g = lane; g < n_groups; g += SYN_WAVE) {
+      float best = -INFINITY;
+      for (int j = 0; j < per; ++j) best = fmaxf(best, c[g * per + j]);
+      grp[g] = best;
+    }
+    wave_sync();
+    // a group stays if fewer than keep_groups others come before it (a larger score, or an equal one at a lower index)
+    for (int g = lane; g < n_groups; g += SYN_WAVE) {
+      int before = 0;
+      for (int o = 0; o < n_groups; ++o) before += (grp[o] > grp[g] || (grp[o] == grp[g] && o < g)) ? 1 : 0;
+      if (before >= keep_groups)
+        for (int j = 0; j < per; ++j) c[g * per + j] = -INFINITY;
+    }
+    wave_sync();
+  }
+  for (int t = 0; t < top; ++t) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += SYN_WAVE) {
+      const float v = c[e];
+      if (v > best) best = v, at = e;      // (a lane meets its experts in rising order)
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, SYN_WAVE);
+      const int oa = __shfl_xor(at, off, SYN_WAVE);
+      if (ob > best || (ob == best && oa < at)) best = ob, at = oa;
+    }
+    if (lane == 0) {
+      if (at >= E) at = t;          // nothing left to choose from: any expert, and no access beyond the table
+      ids[(size_t)tok * top + t] = at;
+      chosen[t] = sc[at];
+      c[at] = -INFINITY;
+    }
+    wave_sync();
+  }
+  if (lane == 0) {
+    float total = 1.f;
+    if (renorm) {
+      total = 0.f;
+      for (int t = 0; t < top; ++t) total += chosen[t];
+    }
+    for (int t = 0; t < top; ++t) weights[(size_t)tok * top + t] = chosen[t] / total;
+  }
+}
+
+SYN_EXPORT int syn_route_scores(const float* logits, const float* correction, int* ids, float* weights, int n_tokens, int E,
+                                int top, int n_groups, int keep_groups, int renorm, hipStream_t stream) {
+  SYN_CHECK(n_tokens > 0, "route_scores: empty input");
+  SYN_CHECK(E > 0 && E <= ROUTE_MAX_EXPERTS, "route_scores: %d experts (at most %d)", E, ROUTE_MAX_EXPERTS);
+  SYN_CHECK(n_groups > 0 && E % n_groups == 0 && keep_groups > 0 && keep_groups <= n_groups,
+            "route_scores: %d experts in %d groups of which %d stay", E, n_groups, keep_groups);
+  SYN_CHECK(top > 0 && top <= ROUTE_MAX_TOP && top <= keep_groups * (E / n_groups),
+            "route_scores: the %d largest of %d groups of %d (at most %d)", top, keep_groups, E / n_groups, ROUTE_MAX_TOP);
+  route_scores_kernel<<<(n_tokens + 3) / 4, 256, 0, stream>>>(logits, correction, ids, weights, n_tokens, E, top, n_groups,
+                                                             keep_groups, renorm);
+  SYN_LAUNCH_CHECK("route_scores");
+  return 0;
+}
+
+// Experts that are the identity: for the places r of seg_start[first] .. seg_start[last] (the segments of the experts
+// first .. last - 1 after the sort), out[o_rows[r]] = weight_of[r] * x[a_rows[r]].  x [*, H] in the engine's type, out
+// [*, H] float.  One workgroup a place of the list; those outside the range leave at once.
+template <typename T>
+__global__ void __launch_bounds__(256) route_identity_kernel(const T* __restrict__ x, float* __restrict__ out,
+                                                             const int* __restrict__ seg_start, int first, int last,
+                                                             const int* __restrict__ a_rows, const int* __restrict__ o_rows,
+                                                             const float* __restrict__ weight_of, int H) {
+  const int r = blockIdx.x;
+  if (r < seg_start[first] || r >= seg_start[last]) return;
+  const T* src = x + (size_t)a_rows[r] * H;
+  float* dst = out + (size_t)o_rows[r] * H;
+  const float w = weight_of[r];
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = w * to_f32<T>(src[i]);
+}
+
+SYN_EXPORT int syn_route_identity(const void* x, int is_f32, float* out, const int* seg_start, int first, int last,
+                                  const int* a_rows, const int* o_rows, const float* weight_of, int places, int H,
+                                  hipStream_t stream) {
+  SYN_CHECK(places > 0 && H > 0 && first >= 0 && last >= first, "route_identity: empty input");
+  if (last == first) return 0;
+  if (is_f32)
+    route_identity_kernel<float><<<places, 256, 0, stream>>>((const float*)x, out, seg_start, first, last, a_rows, o_rows,
+                                                             weight_of, H);
+  else
+    route_identity_kernel<bf16><<<places, 256, 0, stream>>>((const bf16*)x, out, seg_start, first, last, a_rows, o_rows,
+                                                            weight_of, H);
+  SYN_LAUNCH_CHECK("route_identity");
+  return 0;
+}
+
 // ---------------------------------------------------------------- the router's choices as segments
 // P = n_tokens * top pairs (token n, its t-th expert), pair p = n * top + t.  Sorted by expert:
 //   seg_start[e] .. seg_start[e + 1]: the places of expert e;  for a place r:

@@ -507,39 +507,45 @@ SYN_EXPORT int syn_matrix_memory_scan(const float* proj, int width, const float*
 
 // Each head's o divided by its root mean square, times a gain over all heads' values, times sigmoid(gate):
 // one wave for each (token, head).  gate: float rows of gate_stride values (the fused projection from its gate on).
+// silu_first: the gate acts before the norm instead, as o * silu(gate), and the norm sees the gated values.
 template <typename TOut>
 __global__ void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ gain, float eps,
                                       const float* __restrict__ gate, int gate_stride, TOut* __restrict__ out,
-                                      int n_items, int H, int vdim) {
+                                      int n_items, int H, int vdim, int silu_first) {
   const int item = blockIdx.x * (blockDim.x / SYN_WAVE) + threadIdx.x / SYN_WAVE;
   if (item >= n_items) return;
   const int lane = threadIdx.x % SYN_WAVE;
   const int tok = item / H, h = item % H;
   const float* x = o + ((size_t)tok * H + h) * vdim;
-  float ss = 0.f;
-  for (int d = lane; d < vdim; d += SYN_WAVE) ss += x[d] * x[d];
-  const float inv = 1.f / sqrtf(wave_sum(ss) / (float)vdim + eps);
   const float* g = gate ? gate + (size_t)tok * gate_stride + (size_t)h * vdim : nullptr;
+  const bool first = silu_first && g;
+  float ss = 0.f;
   for (int d = lane; d < vdim; d += SYN_WAVE) {
-    float v = x[d] * inv;
+    const float v = first ? x[d] * (g[d] / (1.f + expf(-g[d]))) : x[d];
+    ss += v * v;
+  }
+  const float inv = 1.f / sqrtf(wave_sum(ss) / (float)vdim + eps);
+  for (int d = lane; d < vdim; d += SYN_WAVE) {
+    float v = (first ? x[d] * (g[d] / (1.f + expf(-g[d]))) : x[d]) * inv;
     if (gain) v *= gain[h * vdim + d];
-    if (g) v *= 1.f / (1.f + expf(-g[d]));
+    if (g && !first) v *= 1.f / (1.f + expf(-g[d]));
     out[((size_t)tok * H + h) * vdim + d] = from_f32<TOut>(v);
   }
 }
 
 SYN_EXPORT int syn_head_norm_gate(const float* o, const float* gain, float eps, const float* gate, int gate_stride,
-                                  void* out, int out_is_f32, int n_tokens, int H, int vdim, hipStream_t stream) {
+                                  void* out, int out_is_f32, int n_tokens, int H, int vdim, int silu_first,
+                                  hipStream_t stream) {
   SYN_CHECK(n_tokens > 0 && H > 0 && vdim > 0, "head_norm_gate: empty input");
   SYN_CHECK(gate == nullptr || gate_stride >= H * vdim, "head_norm_gate: gate rows of %d values", gate_stride);
   const int wpb = 4, items = n_tokens * H;
   const int grid = (items + wpb - 1) / wpb;
   if (out_is_f32)
     head_norm_gate_kernel<float><<<grid, wpb * SYN_WAVE, 0, stream>>>(o, gain, eps, gate, gate_stride, (float*)out, items,
-                                                                      H, vdim);
+                                                                      H, vdim, silu_first);
   else
     head_norm_gate_kernel<bf16><<<grid, wpb * SYN_WAVE, 0, stream>>>(o, gain, eps, gate, gate_stride, (bf16*)out, items,
-                                                                     H, vdim);
+                                                                     H, vdim, silu_first);
   SYN_LAUNCH_CHECK("head_norm_gate");
   return 0;
 }

@@ -30,7 +30,7 @@ FLAGS = ["-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-shared", "-fv
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"]
 CORE_SOURCES = ["elementwise.hip", "sampling.hip", "gemm.hip", "attention_f32.hip", "probes.hip", "streams.hip",
-                "attention_window.hip", "matrix_memory.hip", "grouped.hip", "latent.hip", "latent_attention.hip"]
+                "attention_window.hip", "matrix_memory.hip", "grouped.hip", "latent.hip", "latent_attention.hip", "recurrent.hip"]
 RUNTIME_SOURCES = ["runtime.cpp"]
 REF_SOURCES = ["ref/ref_kernels.cpp"]          # the kernels' plain C++ twins (host code)
 ATTN_SOURCE = "attention_bf16.hip"

@@ -139,19 +139,34 @@ def _is_f32(t):
 
 
 # The activations of a gated feed-forward that the kernels apply (codes of gate_activation in csrc/common.h).
-ACTIVATIONS = {"silu": 0, "swish": 0, "gelu_tanh": 1}
+# "swiglu_limit" comes with its bound, as the pair ("swiglu_limit", limit):
+#   g <- min(g, limit), u <- clamp(u, -limit, limit);  g sigmoid(1.702 g) (u + 1)
+ACTIVATIONS = {"silu": 0, "swish": 0, "gelu_tanh": 1, "swiglu_limit": 2}
 
 
 def activation_code(name) -> int:
+    if isinstance(name, (tuple, list)) and len(name) == 2:
+        name = name[0]
     if name not in ACTIVATIONS:
         raise KernelError(f"activation {name!r}: the kernels apply {sorted(set(ACTIVATIONS))}")
     return ACTIVATIONS[name]
 
 
+def _activation_args(activation):
+    """(code, limit) as the entry points take them; an activation with a bound is the pair (name, bound)."""
+    code = activation_code(activation)
+    limit = 0.0
+    if code == ACTIVATIONS["swiglu_limit"]:
+        if not isinstance(activation, (tuple, list)) or not float(activation[1]) > 0.0:
+            raise KernelError("activation 'swiglu_limit' comes with its bound: ('swiglu_limit', limit), limit > 0")
+        limit = float(activation[1])
+    return code, ctypes.c_float(limit)
+
+
 # ----------------------------------------------------------------------------- rows
 
-def embed(table, ids, resid):
-    """resid[n, :] = table[ids[n], :] as float.  table [V, H] bf16|f32 (or bf16 in fragment order, pack_weight: four
+def embed(table, ids, resid, scale=1.0):
+    """resid[n, :] = scale * table[ids[n], :] as float.  table [V, H] bf16|f32 (or bf16 in fragment order, pack_weight: four
     dimensions), ids [N] int32, resid [N, H] f32."""
     if isinstance(table, torch.Tensor) and table.dim() == 4:
         _need(table, "embed.table", _BF16, (None, None, 64, 8))
@@ -161,7 +176,8 @@ def embed(table, ids, resid):
         H, kind = table.shape[1], _is_f32(table)
     _need(ids, "embed.ids", _I32, (None,))
     _need(resid, "embed.resid", _F32, (ids.shape[0], H))
-    _call(load_library("core"), "syn_embed", _ptr(table), kind, _ptr(ids), _ptr(resid), ids.shape[0], H, _stream())
+    _call(load_library("core"), "syn_embed", _ptr(table), kind, _ptr(ids), _ptr(resid), ids.shape[0], H,
+          ctypes.c_float(scale), _stream())
 
 
 def add_rmsnorm(resid, delta, gain, eps, out, rows=None, gain_offset=0.0):
@@ -205,7 +221,7 @@ def swiglu(gate_up, out, activation="silu"):
         raise KernelError(f"swiglu: fused width {I2} is odd")
     _need(out, "swiglu.out", gate_up.dtype, (N, I2 // 2))
     _call(load_library("core"), "syn_swiglu", _ptr(gate_up), _ptr(out), _is_f32(gate_up), N, I2 // 2,
-          activation_code(activation), _stream())
+          *_activation_args(activation), _stream())
 
 
 # ----------------------------------------------------------------------------- matrix product
@@ -290,7 +306,7 @@ def gemm_swiglu(x, w_paired, out, activation="silu"):
                         activation=activation)
         return
     _call(load_library("core"), "syn_gemm_swiglu", _ptr(x), _ptr(w_paired), _ptr(out), M, N, K,
-          activation_code(activation), 1 if packed else 0, _stream())
+          *_activation_args(activation), 1 if packed else 0, _stream())
 
 
 PACKED_BLOCK_ROWS = 16   # the most rows that a product of gemm_packed takes
@@ -370,10 +386,10 @@ def gemm_packed(x, wp, out, paired=False, activation="silu", row_scale=None, res
         out_code = 2 if out.dtype == _F32 else 1
     if row_scale is None and resid_norm is None:
         _call(load_library("core"), "syn_gemm_packed", _ptr(x), _ptr(wp), _ptr(out), out_code,
-              M, N, K, 1 if paired else 0, activation_code(activation), slices, _stream())
+              M, N, K, 1 if paired else 0, *_activation_args(activation), slices, _stream())
         return
     _call(load_library("core"), "syn_gemm_packed_norm", _ptr(x), _ptr(wp), _ptr(out), out_code, M, N, K,
-          1 if paired else 0, activation_code(activation), slices, _ptr(ss), int(groups), int(dim), ctypes.c_float(eps),
+          1 if paired else 0, *_activation_args(activation), slices, _ptr(ss), int(groups), int(dim), ctypes.c_float(eps),
           _ptr(resid), _ptr(xs), _ptr(ss_out), _ptr(gain), _is_f32(gain) if gain is not None else 0,
           ctypes.c_float(gain_offset), _stream())
 
@@ -798,20 +814,28 @@ def streams_start(x, X):
 WINDOW_ATTENTION_MAX_DIM = 640
 
 
-def _check_window_pages(k_pages, v_pages, dtype, nkv, dim, vdim, name):
+def _check_window_pages(k_pages, v_pages, dtype, nkv, dim, vdim, name, v_share=1):
+    if v_share < 1 or nkv % v_share:
+        raise KernelError(f"{name}: {nkv} kv heads in shares of {v_share} value heads")
     _need(k_pages, name + ".k_pages", dtype, (None, nkv, PAGE_TOKENS, dim))
-    _need(v_pages, name + ".v_pages", dtype, (k_pages.shape[0], nkv, vdim, PAGE_TOKENS))
+    _need(v_pages, name + ".v_pages", dtype, (k_pages.shape[0], nkv // v_share, vdim, PAGE_TOKENS))
 
 
 def window_intake(proj, bias, q_out, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps,
-                  n_heads, n_kv_heads, dim, vdim, write_kv=True):
+                  n_heads, n_kv_heads, dim, vdim, write_kv=True, rotation=None, v_share=1):
     """proj [N, width] float: the fused projection [q | k | v | ...]; bias float [>= q, k, v columns] or None.  q and k
     heads get their bias and (with gains, float [dim]) an RMSNorm over the head; q goes to q_out [N, nh * dim], k and v
-    (with its bias) into the pages of sequence tok_seq[n] at position tok_pos[n]."""
+    (with its bias) into the pages of sequence tok_seq[n] at position tok_pos[n].
+    rotation = (cos, sin) float [positions, rot / 2]: the first `rot` values of every q and k head are then turned by
+    the angles of the token's position, value i paired with value i + rot / 2 (the caller sees to it that the tables
+    reach the step's last position).  v_share: there are nkv / v_share value heads (and rows of v in proj)."""
     nh, nkv = n_heads, n_kv_heads
     _need(proj, "window_intake.proj", _F32, (None, None))
     N, width = proj.shape
-    used = (nh + nkv) * dim + nkv * vdim
+    if v_share < 1 or nkv % v_share:
+        raise KernelError(f"window_intake: {nkv} kv heads in shares of {v_share} value heads")
+    nv = nkv // v_share
+    used = (nh + nkv) * dim + nv * vdim
     if width < used:
         raise KernelError(f"window_intake: rows of {width} values do not hold q, k and v ({used})")
     if bias is not None:
@@ -819,8 +843,17 @@ def window_intake(proj, bias, q_out, k_pages, v_pages, page_table, tok_seq, tok_
         if bias.shape[0] < used:
             raise KernelError(f"window_intake: a bias of {bias.shape[0]} values for {used} columns")
     _need(q_out, "window_intake.q_out", (_BF16, _F32), (N, nh * dim))
-    _check_window_pages(k_pages, v_pages, q_out.dtype, nkv, dim, vdim, "window_intake")
+    _check_window_pages(k_pages, v_pages, q_out.dtype, nkv, dim, vdim, "window_intake", v_share)
     _need(page_table, "window_intake.page_table", _I32, (None, None))
+    cos = sin = None
+    rot = 0
+    if rotation is not None and rotation[0] is not None:
+        cos, sin = rotation
+        _need(cos, "window_intake.cos", _F32, (None, None))
+        _need(sin, "window_intake.sin", _F32, tuple(cos.shape))
+        rot = 2 * cos.shape[1]
+        if rot > dim:
+            raise KernelError(f"window_intake: a rotation of {rot} values of heads of {dim}")
     _need(tok_seq, "window_intake.tok_seq", _I32, (N,))
     _need(tok_pos, "window_intake.tok_pos", _I32, (N,))
     if (q_gain is None) != (k_gain is None):
@@ -830,13 +863,15 @@ def window_intake(proj, bias, q_out, k_pages, v_pages, page_table, tok_seq, tok_
         _need(k_gain, "window_intake.k_gain", _F32, (dim,))
     _call(load_library("core"), "syn_window_intake", _ptr(proj), width, _ptr(bias), _ptr(q_out), _ptr(k_pages),
           _ptr(v_pages), _is_f32(q_out), _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos),
-          _ptr(q_gain), _ptr(k_gain), ctypes.c_float(eps), N, nh, nkv, dim, vdim, 1 if write_kv else 0, _stream())
+          _ptr(q_gain), _ptr(k_gain), ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, N, nh, nkv, nv, dim, vdim,
+          1 if write_kv else 0, _stream())
 
 
 def window_attention(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, n_heads, n_kv_heads, dim, vdim,
                      window=0, keep_first=0, sink_one=False, slopes=None, log_bias=None, softcap=0.0, gate=None,
-                     gate_bias=None):
-    """Attention of every token (prompts and single tokens alike) whose query is q [N, nh * dim] over the pages
+                     gate_bias=None, v_share=1):
+    """v_share: that many neighbouring kv heads read the values of one value head (v_pages holds nkv / v_share heads).
+    Attention of every token (prompts and single tokens alike) whose query is q [N, nh * dim] over the pages
     (which already hold the tokens): score = scale q.k [soft cap] - slopes[h] (i - j) - r1[h] ln(1 + r2[h] (i - j))
     with log_bias = (r1, r2) float [nh]; key j is seen by i iff j <= i and (no window or i - j < window or
     j < keep_first); sink_one: one more in the softmax's denominator; gate: a float view [N, >= nh * vdim] with row
@@ -844,7 +879,7 @@ def window_attention(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, sca
     nh, nkv = n_heads, n_kv_heads
     _need(q, "window_attention.q", (_BF16, _F32), (None, nh * dim))
     N = q.shape[0]
-    _check_window_pages(k_pages, v_pages, q.dtype, nkv, dim, vdim, "window_attention")
+    _check_window_pages(k_pages, v_pages, q.dtype, nkv, dim, vdim, "window_attention", v_share)
     _need(page_table, "window_attention.page_table", _I32, (None, None))
     _need(tok_seq, "window_attention.tok_seq", _I32, (N,))
     _need(tok_pos, "window_attention.tok_pos", _I32, (N,))
@@ -867,7 +902,7 @@ def window_attention(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, sca
           _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos), _ptr(gate), gate_stride,
           _ptr(gate_bias if gate is not None else None), _ptr(out), ctypes.c_float(scale), N, nh, nkv, dim, vdim,
           _ptr(slopes), _ptr(r1), _ptr(r2), ctypes.c_float(float(softcap or 0.0)), int(window or 0), int(keep_first or 0),
-          1 if sink_one else 0, _stream())
+          1 if sink_one else 0, int(v_share), _stream())
 
 
 WINDOW_PREFILL_MAX_DIM = 128
@@ -880,7 +915,7 @@ def window_prefill_takes(dim, vdim) -> bool:
 
 def window_attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past, out, scale, n_heads, n_kv_heads,
                                   dim, vdim, window=0, keep_first=0, sink_one=False, slopes=None, log_bias=None,
-                                  softcap=0.0, gate=None, gate_bias=None):
+                                  softcap=0.0, gate=None, gate_bias=None, v_share=1):
     """window_attention for the new tokens of each sequence of a step in bf16, on the matrix cores: seq_start [B + 1]
     offsets of the sequences' new tokens in q, seq_past [B] tokens cached before (the pages already hold the new
     ones).  Scores and weights are 32-bit; a weight meets V as two bf16 numbers (16 bits of mantissa)."""
@@ -889,7 +924,7 @@ def window_attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, se
         raise KernelError(f"window_attention_prefill: head sizes {dim} and {vdim} (multiples of 16 up to {WINDOW_PREFILL_MAX_DIM})")
     _need(q, "window_attention_prefill.q", _BF16, (None, nh * dim))
     N = q.shape[0]
-    _check_window_pages(k_pages, v_pages, _BF16, nkv, dim, vdim, "window_attention_prefill")
+    _check_window_pages(k_pages, v_pages, _BF16, nkv, dim, vdim, "window_attention_prefill", v_share)
     _need(page_table, "window_attention_prefill.page_table", _I32, (None, None))
     _need(seq_start, "window_attention_prefill.seq_start", _I32, (None,))
     B = seq_start.shape[0] - 1
@@ -913,7 +948,7 @@ def window_attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, se
           _ptr(page_table), page_table.shape[1], _ptr(seq_start), _ptr(seq_past), B, N, _ptr(gate), gate_stride,
           _ptr(gate_bias if gate is not None else None), _ptr(out), ctypes.c_float(scale), nh, nkv, dim, vdim,
           _ptr(slopes), _ptr(r1), _ptr(r2), ctypes.c_float(float(softcap or 0.0)), int(window or 0), int(keep_first or 0),
-          1 if sink_one else 0, _stream())
+          1 if sink_one else 0, int(v_share), _stream())
 
 
 def _float_rows_view(t, name, n_rows, n_cols):
@@ -973,9 +1008,10 @@ def matrix_memory_scan(proj, i_bias, f_bias, gate_cap, q_scale, state, seq_start
           _ptr(seq_slot), B, _ptr(out), H, dim, vdim, 1 if chunked else 0, N, _ptr(work), _stream())
 
 
-def head_norm_gate(o, gain, eps, gate, out, n_heads, vdim):
+def head_norm_gate(o, gain, eps, gate, out, n_heads, vdim, silu_first=False):
     """out[n, h] = o[n, h] / rms(o[n, h]) * gain[h] * sigmoid(gate[n, h]): o [N, H * vdim] float, gain float [H * vdim]
-    or None, gate a float view [N, >= H * vdim] (see _float_rows_view) or None, out [N, H * vdim] bf16 or float."""
+    or None, gate a float view [N, >= H * vdim] (see _float_rows_view) or None, out [N, H * vdim] bf16 or float.
+    silu_first: the gate comes before the norm, x = o * silu(gate), out = x / rms(x) * gain."""
     _need(o, "head_norm_gate.o", _F32, (None, n_heads * vdim))
     N = o.shape[0]
     if gain is not None:
@@ -983,7 +1019,110 @@ def head_norm_gate(o, gain, eps, gate, out, n_heads, vdim):
     stride = _float_rows_view(gate, "head_norm_gate.gate", N, n_heads * vdim) if gate is not None else 0
     _need(out, "head_norm_gate.out", (_BF16, _F32), (N, n_heads * vdim))
     _call(load_library("core"), "syn_head_norm_gate", _ptr(o), _ptr(gain), ctypes.c_float(eps), _ptr(gate), stride,
-          _ptr(out), _is_f32(out), N, n_heads, vdim, _stream())
+          _ptr(out), _is_f32(out), N, n_heads, vdim, 1 if silu_first else 0, _stream())
+
+
+# ----------------------------------------------------------------------------- short convolutions and scans over a state
+
+SHORT_CONV_MAX_TAPS = 16
+SCAN_MAX_ROWS = 256       # rows of a head's state: the state space's N, the delta rule's key size
+
+
+def _step_seqs(name, seq_start, seq_slot):
+    _need(seq_start, name + ".seq_start", _I32, (None,))
+    B = seq_start.shape[0] - 1
+    _need(seq_slot, name + ".seq_slot", _I32, (B,))
+    return B
+
+
+def short_conv(u, weight, bias, state, tok_seq, tok_pos, seq_start, seq_past, seq_slot, out, silu=False):
+    """A causal convolution over each sequence's own tokens, one filter a channel:
+    out[t, c] = act(bias[c] + sum_j weight[c, j] u[t - taps + 1 + j, c]), zeros before a sequence's first token.
+    u: a float view [N, C] whose rows may be pieces of longer rows (columns of a fused projection); weight float
+    [C, taps]; bias float [C] or None; state float [rows, taps - 1, C]: the last taps - 1 inputs of the sequence in row
+    seq_slot[b] (a negative slot: the last row), read for the tokens before this step and written for the next one;
+    out float [N, C]."""
+    _need(weight, "short_conv.weight", _F32, (None, None))
+    C, taps = weight.shape
+    N = tok_seq.shape[0]
+    stride = _float_rows_view(u, "short_conv.u", N, C)
+    if not 1 <= taps <= SHORT_CONV_MAX_TAPS:
+        raise KernelError(f"short_conv: {taps} taps (1 to {SHORT_CONV_MAX_TAPS})")
+    if bias is not None:
+        _need(bias, "short_conv.bias", _F32, (C,))
+    _need(state, "short_conv.state", _F32, (None, max(taps - 1, 0), C))
+    _need(tok_seq, "short_conv.tok_seq", _I32, (N,))
+    _need(tok_pos, "short_conv.tok_pos", _I32, (N,))
+    B = _step_seqs("short_conv", seq_start, seq_slot)
+    _need(seq_past, "short_conv.seq_past", _I32, (B,))
+    _need(out, "short_conv.out", _F32, (N, C))
+    _call(load_library("core"), "syn_short_conv", _ptr(u), stride, _ptr(weight), _ptr(bias), 1 if silu else 0, _ptr(state),
+          state.shape[0], _ptr(tok_seq), _ptr(tok_pos), _ptr(seq_start), _ptr(seq_past), _ptr(seq_slot), _ptr(out), N, B, C,
+          taps, _stream())
+
+
+def state_space_scan(xbc, dt, dt_bias, a_log, d_skip, state, seq_start, seq_slot, out, n_heads, vdim, n_state, n_groups):
+    """The state space with a scalar decay a head over the new tokens of every sequence of the step, in order:
+        step = softplus(dt + dt_bias[h]);  S <- exp(-exp(a_log[h]) step) S + step B x^T;  y = S^T C + d_skip[h] x
+    xbc float [N, H * vdim + 2 G * n_state]: x, B and C (head h reads group h // (H / G)); dt a float view [N, >= H];
+    state float [rows, H, n_state, vdim] (row seq_slot[b]; a negative slot: the last row); out float [N, H * vdim]."""
+    H, G = n_heads, n_groups
+    if G <= 0 or H % G:
+        raise KernelError(f"state_space_scan: {H} heads do not divide into {G} groups")
+    if n_state > SCAN_MAX_ROWS:
+        raise KernelError(f"state_space_scan: a state of {n_state} rows (at most {SCAN_MAX_ROWS})")
+    _need(xbc, "state_space_scan.xbc", _F32, (None, H * vdim + 2 * G * n_state))
+    N = xbc.shape[0]
+    stride = _float_rows_view(dt, "state_space_scan.dt", N, H)
+    for name, t in (("dt_bias", dt_bias), ("a_log", a_log), ("d_skip", d_skip)):
+        _need(t, f"state_space_scan.{name}", _F32, (H,))
+    _need(state, "state_space_scan.state", _F32, (None, H, n_state, vdim))
+    B = _step_seqs("state_space_scan", seq_start, seq_slot)
+    _need(out, "state_space_scan.out", _F32, (N, H * vdim))
+    _call(load_library("core"), "syn_state_space_scan", _ptr(xbc), _ptr(dt), stride, _ptr(dt_bias), _ptr(a_log),
+          _ptr(d_skip), _ptr(state), state.shape[0], _ptr(seq_start), _ptr(seq_slot), B, _ptr(out), H, vdim, n_state, G,
+          _stream())
+
+
+def channel_delta_scan(qkv, beta, a, a_bias, a_log, q_scale, unit_eps, state, seq_start, seq_slot, out, n_heads,
+                       n_key_heads, dim, vdim):
+    """The delta rule with a decay for every key channel over the new tokens of every sequence of the step, in order.
+    With q and k made unit vectors (x / sqrt(sum x^2 + unit_eps); q also times q_scale), b = sigmoid(beta) and
+    g = exp(-exp(a_log[h]) softplus(a + a_bias)) for each (head, key channel):
+        S <- diag(g) S;  u = b (v - S^T k);  S <- S + k u^T;  o = S^T q
+    qkv float [N, 2 K * dim + H * vdim]: q and k of the K key heads (head h reads key head h // (H / K)), v; beta a
+    float view [N, >= H]; a a float view [N, >= H * dim]; a_bias float [H * dim]; a_log float [H]; state float
+    [rows, H, dim, vdim] (row seq_slot[b]; a negative slot: the last row); out float [N, H * vdim]."""
+    H, K = n_heads, n_key_heads
+    if K <= 0 or H % K:
+        raise KernelError(f"channel_delta_scan: {H} heads do not divide into {K} key heads")
+    if dim > SCAN_MAX_ROWS:
+        raise KernelError(f"channel_delta_scan: keys of {dim} values (at most {SCAN_MAX_ROWS})")
+    _need(qkv, "channel_delta_scan.qkv", _F32, (None, 2 * K * dim + H * vdim))
+    N = qkv.shape[0]
+    stride = _float_rows_view(beta, "channel_delta_scan.beta", N, H)
+    a_stride = _float_rows_view(a, "channel_delta_scan.a", N, H * dim)
+    _need(a_bias, "channel_delta_scan.a_bias", _F32, (H * dim,))
+    _need(a_log, "channel_delta_scan.a_log", _F32, (H,))
+    _need(state, "channel_delta_scan.state", _F32, (None, H, dim, vdim))
+    B = _step_seqs("channel_delta_scan", seq_start, seq_slot)
+    _need(out, "channel_delta_scan.out", _F32, (N, H * vdim))
+    _call(load_library("core"), "syn_channel_delta_scan", _ptr(qkv), _ptr(beta), stride, _ptr(a), a_stride, _ptr(a_bias),
+          _ptr(a_log),
+          ctypes.c_float(q_scale), ctypes.c_float(unit_eps), _ptr(state), state.shape[0], _ptr(seq_start), _ptr(seq_slot), B,
+          _ptr(out), H, K, dim, vdim, _stream())
+
+
+def diff_heads(a, out, lam, eps, post, n_kv_heads, heads_per_kv, vdim):
+    """Two softmax maps over the same values joined: a [N, G * 2 * R * vdim] holds, for each of the G kv heads, the R
+    heads' results of the first map and then of the second; out [N, G * R * vdim] = rms_norm(a1 - lam a2) * post for
+    each head (the norm over the head's vdim values, eps inside the root, no gain)."""
+    G, R = n_kv_heads, heads_per_kv
+    _need(a, "diff_heads.a", (_BF16, _F32), (None, G * 2 * R * vdim))
+    N = a.shape[0]
+    _need(out, "diff_heads.out", a.dtype, (N, G * R * vdim))
+    _call(load_library("core"), "syn_diff_heads", _ptr(a), _ptr(out), _is_f32(a), ctypes.c_float(lam), ctypes.c_float(eps),
+          ctypes.c_float(post), N, G, R, vdim, _stream())
 
 
 # ----------------------------------------------------------------------------- sampling
@@ -1163,6 +1302,43 @@ def route_sort(ids, weights, n_experts):
     _call(load_library("core"), "syn_route_sort", _ptr(ids), _ptr(weights), _ptr(seg), _ptr(lists[0]), _ptr(lists[1]),
           _ptr(lists[2]), _ptr(weight_of), N, top, n_experts, _stream())
     return seg, lists[0], lists[1], lists[2], weight_of
+
+
+def route_scores(logits, correction, ids, weights, n_groups=1, keep_groups=1, renorm=False):
+    """A router that scores every expert: s = softmax(logits [N, E] float) over all E; the choice is made on
+    s + correction [E] among the members of the keep_groups best of n_groups equal groups of neighbours (a group's
+    score: its largest choice score); ids [N, top] int32 the chosen (largest first, the lower index of equal ones),
+    weights [N, top] float their s, divided by their sum with renorm."""
+    _need(logits, "route_scores.logits", _F32, (None, None))
+    N, E = logits.shape
+    if correction is not None:
+        _need(correction, "route_scores.correction", _F32, (E,))
+    _need(ids, "route_scores.ids", _I32, (N, None))
+    top = ids.shape[1]
+    _need(weights, "route_scores.weights", _F32, (N, top))
+    if E > ROUTE_MAX_EXPERTS or n_groups <= 0 or E % n_groups or not 0 < keep_groups <= n_groups:
+        raise KernelError(f"route_scores: {E} experts (at most {ROUTE_MAX_EXPERTS}) in {n_groups} groups, {keep_groups} kept")
+    if not 0 < top <= min(keep_groups * (E // n_groups), ROUTE_MAX_TOP):
+        raise KernelError(f"route_scores: the {top} largest of {keep_groups} groups of {E // n_groups} (at most {ROUTE_MAX_TOP})")
+    _call(load_library("core"), "syn_route_scores", _ptr(logits), _ptr(correction), _ptr(ids), _ptr(weights), N, E, top,
+          int(n_groups), int(keep_groups), 1 if renorm else 0, _stream())
+
+
+def route_identity(x, out, seg, first, last, a_rows, o_rows, weight_of):
+    """Experts first .. last - 1 of a sorted choice (route_sort) are the identity: out[o_rows[r]] = weight_of[r] *
+    x[a_rows[r]] for the places r of their segments.  x [*, H] in the engine's type, out [*, H] float."""
+    _need(x, "route_identity.x", (_BF16, _F32), (None, None))
+    H = x.shape[1]
+    _need(out, "route_identity.out", _F32, (None, H))
+    _need(seg, "route_identity.seg", _I32, (None,))
+    if not 0 <= first <= last < seg.shape[0]:
+        raise KernelError(f"route_identity: experts {first} .. {last} of {seg.shape[0] - 1}")
+    _need(a_rows, "route_identity.a_rows", _I32, (None,))
+    P = a_rows.shape[0]
+    _need(o_rows, "route_identity.o_rows", _I32, (P,))
+    _need(weight_of, "route_identity.weight_of", _F32, (P,))
+    _call(load_library("core"), "syn_route_identity", _ptr(x), _is_f32(x), _ptr(out), _ptr(seg), int(first), int(last),
+          _ptr(a_rows), _ptr(o_rows), _ptr(weight_of), P, H, _stream())
 
 
 def pack_expert_weights(w):

@@ -2,5 +2,6 @@ from .decoder import DecoderModel, LayerRun, TokenEmbedding, OutputHead
 from .qwen3 import build_qwen3
 from .bizipel import build_bizipel
 from .kamivik import build_kamivik
+from .repolix import build_repolix
 
-__all__ = ["DecoderModel", "LayerRun", "TokenEmbedding", "OutputHead", "build_qwen3", "build_bizipel", "build_kamivik"]
+__all__ = ["DecoderModel", "LayerRun", "TokenEmbedding", "OutputHead", "build_qwen3", "build_bizipel", "build_kamivik", "build_repolix"]

@@ -30,11 +30,11 @@ class LayerRun:
 
 
 class TokenEmbedding(Part):
-    """x[n, :] = E[id[n], :] (crates/synaptix-ops/src/embed/token_embed.rs:4-15)."""
+    """x[n, :] = scale * E[id[n], :] (crates/synaptix-ops/src/embed/token_embed.rs:4-15; the reference has no scale)."""
     capturable = True
 
-    def __init__(self, name: str, vocab: int, hidden: int):
-        self.name, self.vocab, self.hidden = name, vocab, hidden
+    def __init__(self, name: str, vocab: int, hidden: int, scale: float = 1.0):
+        self.name, self.vocab, self.hidden, self.scale = name, vocab, hidden, float(scale)
         self.table = None
 
     def tensor_specs(self):
@@ -45,7 +45,10 @@ class TokenEmbedding(Part):
 
     def forward(self, ids):
         resid = torch.empty((ids.shape[0], self.hidden), dtype=torch.float32, device=ids.device)
-        ops.embed(self.table.data, ids, resid)
+        if self.scale == 1.0:
+            ops.embed(self.table.data, ids, resid)
+        else:
+            ops.embed(self.table.data, ids, resid, self.scale)
         return resid
 
 

@@ -44,6 +44,7 @@ class KvNeed:
     window: Optional[int] = None      # None: all keys
     v_dim: Optional[int] = None       # size of a value where it differs from the keys' (None: head_dim)
     keep_first: int = 0               # with a window: the first keys of a sequence that stay visible for good
+    v_heads: Optional[int] = None     # value heads where several kv heads read the values of one (None: kv_heads)
 
 
 def flat_needs(need) -> tuple:

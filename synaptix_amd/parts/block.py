@@ -29,39 +29,70 @@ def _norm_input(norm, delta):
 
 
 class PreNormBlock(Block):
+    """x <- x + s1 * mixer(norm1(x));  x <- x + s2 * ff(norm2(x)).  scale_prefix: the results are multiplied channel by
+    channel by the tensors scale_prefix + "ls1" and "ls2" ([hidden]; None: no scales).  A layer may have no
+    feed-forward (norm2 and feed_forward None): it is its first half only."""
     takes_deferred_product = True
 
-    def __init__(self, norm1, mixer, norm2, feed_forward):
+    def __init__(self, norm1, mixer, norm2=None, feed_forward=None, scale_prefix: str | None = None,
+                 scale_names=("ls1", "ls2"), hidden: int | None = None):
+        if (norm2 is None) != (feed_forward is None):
+            raise ValueError("the second norm and the feed-forward come together")
+        if scale_prefix is not None and hidden is None:
+            raise ValueError("channel scales need the width of the residual")
         self.norm1, self.mixer, self.norm2, self.feed_forward = norm1, mixer, norm2, feed_forward
+        self.scale_prefix, self.scale_names, self.hidden = scale_prefix, tuple(scale_names), hidden
+        self.scales = [None, None]
 
     def _parts(self):
-        return (self.norm1, self.mixer, self.norm2, self.feed_forward)
+        return tuple(p for p in (self.norm1, self.mixer, self.norm2, self.feed_forward) if p is not None)
+
+    def _scale_names(self):
+        if self.scale_prefix is None:
+            return []
+        return [self.scale_prefix + n for n in self.scale_names[:2 if self.feed_forward is not None else 1]]
 
     @property
     def capturable(self):
         return all(getattr(p, "capturable", False) for p in self._parts())
 
     def tensor_specs(self):
+        from ..weights.source import TensorSpec
         specs = {}
         for p in self._parts():
             specs.update(p.tensor_specs())
+        specs.update({n: TensorSpec((self.hidden,), "gain") for n in self._scale_names()})
         return specs
 
     def load(self, get):
         for p in self._parts():
             p.load(get)
+        for i, n in enumerate(self._scale_names()):
+            self.scales[i] = get(n).float().contiguous()
 
     def check(self, dtype):
         for p in self._parts():
             p.check(dtype)
 
+    def _scaled(self, delta, scale):
+        """A sublayer's result with its channels' scales, left for whoever adds the residual next."""
+        from .linear import ChannelScaledDeltas, SummedDeltas
+        if scale is None:
+            return delta
+        terms = delta.terms if isinstance(delta, SummedDeltas) else [delta]
+        return ChannelScaledDeltas([(t, scale) for t in terms])
+
     def forward(self, resid, pending, ctx, cache, owner=True):
         # a norm may hand on rows whose last step a product finishes, and take a product that has not been run
         # (parts.linear.ScaledRows, DeferredProduct); parts that do not say they take them get plain tensors
         h = self.norm1.add_apply(resid, _norm_input(self.norm1, pending), ctx.act_dtype)
-        a = self.mixer.forward(h if self.mixer.takes_scaled_rows else as_rows(h), ctx, cache, owner)
+        a = self._scaled(self.mixer.forward(h if self.mixer.takes_scaled_rows else as_rows(h), ctx, cache, owner),
+                         self.scales[0])
+        if self.feed_forward is None:
+            return a
         h2 = self.norm2.add_apply(resid, _norm_input(self.norm2, a), ctx.act_dtype)
-        return self.feed_forward.forward(h2 if self.feed_forward.takes_scaled_rows else as_rows(h2), ctx)
+        return self._scaled(self.feed_forward.forward(h2 if self.feed_forward.takes_scaled_rows else as_rows(h2), ctx),
+                            self.scales[1])
 
 
 class HyperConnectionBlock(Block):

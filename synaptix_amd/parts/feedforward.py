@@ -73,69 +73,135 @@ class GatedMlp(FeedForward):
 
 
 class RoutedExperts(FeedForward):
-    """A mixture of small ungated experts: each token goes through the `top` experts whose router logits are largest,
+    """A mixture of small experts: each token goes through `top` of them, chosen by a router, and gets the weighted sum
+    of their results.
 
-        z = W_router h + b (32-bit sums of the framework's own product);   chosen: the `top` largest z;
-        weights: softmax over the chosen logits only
-        y = sum_chosen weight_e * W_down[e] act(W_up[e] h)
+    The router (32-bit sums of the framework's own product z = W_router h), one of
+        "top_logits"  the `top` largest z + bias; weights: softmax over the chosen logits only
+        "scores"      s = softmax(z) over all router outputs; the choice is made on s + correction among the members of
+                      the `keep_groups` best of `n_groups` equal groups of neighbours (a group's score: its largest choice
+                      score); weights: the chosen s themselves (`renorm`: divided by their sum)
+    The experts, one of
+        ungated       W_down act(W_up h), act the exact GELU
+        gated         W_down act2(W_gate h, W_up h) with an activation of the gated products (ops.ACTIVATIONS; one with a
+                      bound as the pair (name, bound))
+    `identity`: the router's last `identity` outputs stand for experts without tensors whose result is h itself.
+    `shared`: a feed-forward that every token passes as well (its result is a second term of the sum).
 
     The tokens are sorted by expert on the device (no count comes back to the host), and each expert's rows meet its
     matrices in one launch for all experts (ops.experts_product).  Returns the `top` weighted results of every token
-    as partial sums [top, N, hidden], which whoever adds the residual sums up.
-    Tensors: prefix + "e<j>.up" [ff, hidden], "e<j>.down" [hidden, ff], "router" [experts, hidden], "router.b"."""
+    as partial sums [top, N, hidden], which whoever adds the residual sums up (with `shared`: parts.SummedDeltas of
+    those and the shared result).
+    Tensors: prefix + "e<j>.up" [ff, hidden], "e<j>.down" [hidden, ff] (gated: "e<j>.gate" too), "router"
+    [experts + identity, hidden], "router.b" or "correction"; `names` renames them."""
     takes_scaled_rows = False
     capturable = True
 
-    ACTIVATIONS = ("gelu",)       # the exact (erf) form, the products' epilogue
+    ACTIVATIONS = ("gelu",)       # of ungated experts: the exact (erf) form, the products' epilogue
+    ROUTERS = ("top_logits", "scores")
 
-    def __init__(self, prefix: str, hidden: int, ff: int, n_experts: int, top: int, activation: str = "gelu",
-                 router_bias: bool = True, names=("e{}.up", "e{}.down", "router", "router.b")):
-        if activation not in self.ACTIVATIONS:
+    def __init__(self, prefix: str, hidden: int, ff: int, n_experts: int, top: int, activation="gelu",
+                 router_bias: bool = True, names=None, *, gated: bool = False, router: str = "top_logits",
+                 n_groups: int = 1, keep_groups: int = 1, renorm: bool = False, identity: int = 0, shared=None):
+        if router not in self.ROUTERS:
+            raise ValueError(f"{prefix}: router {router!r} (one of {self.ROUTERS})")
+        if gated:
+            try:
+                ops.activation_code(activation)
+            except ops.KernelError as e:
+                raise ValueError(f"{prefix}: {e}") from None
+        elif activation not in self.ACTIVATIONS:
             raise ValueError(f"{prefix}: activation {activation!r} (the experts' products apply {self.ACTIVATIONS})")
-        if not 0 < top <= n_experts:
-            raise ValueError(f"{prefix}: the {top} largest of {n_experts} experts")
+        total = n_experts + int(identity)
+        if not 0 < top <= total or n_experts < 0 or identity < 0:
+            raise ValueError(f"{prefix}: the {top} largest of {n_experts} experts and {identity} identities")
+        if router == "scores" and (n_groups <= 0 or total % n_groups or not 0 < keep_groups <= n_groups
+                                   or top > keep_groups * (total // n_groups)):
+            raise ValueError(f"{prefix}: {total} router outputs in {n_groups} groups, {keep_groups} kept, {top} chosen")
+        if identity and router != "scores":
+            raise ValueError(f"{prefix}: identity experts come with the router that scores all outputs")
         self.prefix, self.hidden, self.ff, self.n_experts, self.top = prefix, hidden, ff, n_experts, top
-        self.router_bias, self.names = bool(router_bias), tuple(names)
+        self.activation, self.gated, self.router = activation, bool(gated), router
+        self.n_groups, self.keep_groups, self.renorm, self.identity = int(n_groups), int(keep_groups), bool(renorm), int(identity)
+        self.total, self.shared = total, shared
+        self.router_bias = bool(router_bias)
+        if names is None:
+            names = ("e{}.up", "e{}.down", "router", "correction" if router == "scores" else "router.b", "e{}.gate")
+        self.names = tuple(names)
         self.w_up = self.w_down = self.w_router = self.b_router = None
 
+    @property
+    def capturable(self):
+        return self.shared is None or bool(getattr(self.shared, "capturable", False))
+
     def tensor_specs(self):
-        p, (up, down, router, bias) = self.prefix, self.names
-        specs = {p + router: TensorSpec((self.n_experts, self.hidden))}
+        p, (up, down, router, bias) = self.prefix, self.names[:4]
+        specs = {p + router: TensorSpec((self.total, self.hidden))}
         if self.router_bias:
-            specs[p + bias] = TensorSpec((self.n_experts,), "bias")
+            specs[p + bias] = TensorSpec((self.total,), "bias")
         for e in range(self.n_experts):
+            if self.gated:
+                specs[p + self.names[4].format(e)] = TensorSpec((self.ff, self.hidden))
             specs[p + up.format(e)] = TensorSpec((self.ff, self.hidden))
             specs[p + down.format(e)] = TensorSpec((self.hidden, self.ff))
+        if self.shared is not None:
+            specs.update(self.shared.tensor_specs())
         return specs
 
     def load(self, get):
-        p, (up, down, router, bias) = self.prefix, self.names
+        p, (up, down, router, bias) = self.prefix, self.names[:4]
         # every expert's matrices kept once: in fragment order where type and sizes allow, else in plain rows
-        w_up = torch.stack([get(p + up.format(e)) for e in range(self.n_experts)]).contiguous()
-        packed = ops.pack_expert_weights(w_up)
-        self.w_up = w_up if packed is None else packed
-        del w_up, packed
-        w_down = torch.stack([get(p + down.format(e)) for e in range(self.n_experts)]).contiguous()
-        packed = ops.pack_expert_weights(w_down)
-        self.w_down = w_down if packed is None else packed
+        if self.n_experts:
+            if self.gated:      # an expert's gate rows, then its up rows: one product for both
+                w_up = torch.stack([torch.cat([get(p + self.names[4].format(e)), get(p + up.format(e))], 0)
+                                    for e in range(self.n_experts)]).contiguous()
+            else:
+                w_up = torch.stack([get(p + up.format(e)) for e in range(self.n_experts)]).contiguous()
+            packed = ops.pack_expert_weights(w_up)
+            self.w_up = w_up if packed is None else packed
+            del w_up, packed
+            w_down = torch.stack([get(p + down.format(e)) for e in range(self.n_experts)]).contiguous()
+            packed = ops.pack_expert_weights(w_down)
+            self.w_down = w_down if packed is None else packed
         self.w_router = Matrix(get(p + router))
         self.b_router = get(p + bias).float().contiguous() if self.router_bias else None
+        if self.shared is not None:
+            self.shared.load(get)
 
     def check(self, dtype):
-        if self.n_experts > ops.ROUTE_MAX_EXPERTS or self.top > ops.ROUTE_MAX_TOP:
-            raise ValueError(f"{self.prefix}: {self.top} of {self.n_experts} experts "
+        if self.total > ops.ROUTE_MAX_EXPERTS or self.top > ops.ROUTE_MAX_TOP:
+            raise ValueError(f"{self.prefix}: {self.top} of {self.total} experts "
                              f"(at most {ops.ROUTE_MAX_TOP} of {ops.ROUTE_MAX_EXPERTS})")
+        if self.shared is not None:
+            self.shared.check(dtype)
 
     def forward(self, h, ctx):
         h = as_rows(h)
         N, dev = h.shape[0], h.device
         ids = torch.empty((N, self.top), dtype=torch.int32, device=dev)
         weights = torch.empty((N, self.top), dtype=torch.float32, device=dev)
-        ops.route_topk(linear(h, self.w_router, torch.float32), self.b_router, ids, weights)
-        seg, tok_of, pair_of, part_of, weight_of = ops.route_sort(ids, weights, self.n_experts)
-        mid = torch.empty((N * self.top, self.ff), dtype=h.dtype, device=dev)
-        ops.experts_product(h, self.w_up, mid, seg, tok_of, pair_of, gelu=True)
+        logits = linear(h, self.w_router, torch.float32)
+        if self.router == "scores":
+            ops.route_scores(logits, self.b_router, ids, weights, self.n_groups, self.keep_groups, self.renorm)
+        else:
+            ops.route_topk(logits, self.b_router, ids, weights)
+        seg, tok_of, pair_of, part_of, weight_of = ops.route_sort(ids, weights, self.total)
         y = torch.empty((self.top, N, self.hidden), dtype=torch.float32, device=dev)
-        ops.experts_product(mid, self.w_down, y.view(self.top * N, self.hidden), seg, pair_of, part_of,
-                            row_weight=weight_of)
+        if self.n_experts:
+            real = seg[:self.n_experts + 1]          # the experts with matrices come first
+            mid = torch.empty((N * self.top, self.ff), dtype=h.dtype, device=dev)
+            if self.gated:
+                both = torch.empty((N * self.top, 2 * self.ff), dtype=h.dtype, device=dev)
+                ops.experts_product(h, self.w_up, both, real, tok_of, pair_of)
+                ops.swiglu(both, mid, self.activation)
+            else:
+                ops.experts_product(h, self.w_up, mid, real, tok_of, pair_of, gelu=True)
+            ops.experts_product(mid, self.w_down, y.view(self.top * N, self.hidden), real, pair_of, part_of,
+                                row_weight=weight_of)
+        if self.identity:
+            ops.route_identity(h, y.view(self.top * N, self.hidden), seg, self.n_experts, self.total, tok_of, part_of,
+                               weight_of)
+        if self.shared is not None:
+            from .linear import SummedDeltas
+            return SummedDeltas([y, self.shared.forward(h, ctx)])
         return y

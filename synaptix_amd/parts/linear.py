@@ -140,9 +140,25 @@ class ChannelScaledDeltas:
         return total
 
 
+class SummedDeltas:
+    """A sublayer's result as several terms that have not been added yet (routed experts and an expert that every token
+    passes), each a float tensor [N, hidden] or partial sums [P, N, hidden] (or a product that has not been run).  A
+    block that scales its sublayers' results by channel hands the terms on, each with the scales
+    (ChannelScaledDeltas); everything else asks for `run()`, the sum as one tensor."""
+
+    def __init__(self, terms):
+        self.terms = [as_delta(t) for t in terms]
+        self.shape = tuple(self.terms[0].shape[-2:])
+
+    def run(self):
+        return ChannelScaledDeltas([(t, None) for t in self.terms]).run()
+
+
 def as_delta(d):
     """The delta of the residual rows as a tensor (or None), whatever form it arrives in."""
-    return d.run() if isinstance(d, (DeferredProduct, WeightedDeltas, StreamsWrite, ChannelScaledDeltas)) else d
+    if isinstance(d, (DeferredProduct, WeightedDeltas, StreamsWrite, ChannelScaledDeltas, SummedDeltas)):
+        return d.run()
+    return d
 
 
 def deferred_product(x, w):

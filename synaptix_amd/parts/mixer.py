@@ -295,6 +295,116 @@ class GatedWindowAttention(Mixer):
         return WeightedDeltas([(y, 1.0, self.b_o)]) if self.b_o is not None else y
 
 
+class DifferentialAttention(Mixer):
+    """Grouped-query attention in two softmax maps over the same values, joined by a difference:
+
+        q [heads x 2 x dim], k [kv_heads x 2 x dim] (head by head: map 1, map 2), v [kv_heads x vdim];
+        each of q, k, v passes a short causal convolution over time (one filter a channel, no activation);
+        the position scheme turns the first values of every map's q and k;
+        a_m = softmax_j(scale q_m . k_m) v over the keys j with 0 <= i - j (< window), m = 1, 2;
+        lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff  (one number for the layer)
+        o = rms_norm(a_1 - lambda a_2) (1 - diff)  per head over its vdim values, no gain;   W_o on the heads.
+
+    It runs as grouped-query attention with 2 heads x 2 kv_heads of `dim` whose kv heads share their values in pairs
+    (KvNeed.v_heads): the query rows are kept in the order (kv head, map, head of the group), so that a head's two maps
+    read the key heads 2 g and 2 g + 1 of its group g.  The cache holds each token's keys for both maps, its values
+    once, and the convolutions' last taps - 1 inputs.  Scores, weights, the rotation and the norm are 32-bit.
+
+    Tensor names: prefix + "q", "k", "v" (+ ".conv" [channels, taps]), "lq1", "lk1", "lq2", "lk2" [dim], "o"."""
+    takes_scaled_rows = False
+    capturable = True
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "conv": ".conv", "lq1": "lq1", "lk1": "lk1", "lq2": "lq2", "lk2": "lk2"}
+
+    def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, dim: int, v_dim: int, taps: int, *,
+                 diff: float, norm_eps: float, position: Position | None = None, scale: float | None = None,
+                 window: int | None = None, names: dict | None = None):
+        if n_kv_heads <= 0 or n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} heads do not divide into {n_kv_heads} kv heads")
+        self.prefix, self.hidden = prefix, hidden
+        self.nh, self.nkv, self.dim, self.vdim, self.taps = n_heads, n_kv_heads, dim, v_dim, taps
+        self.diff, self.norm_eps = float(diff), float(norm_eps)
+        self.position = position or NoPosition()
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(dim)
+        self.window = window
+        self.names = dict(self.NAMES, **(names or {}))
+        self.channels = (2 * n_heads + 2 * n_kv_heads) * dim + n_kv_heads * v_dim
+        self.w_in = self.w_o = self.conv = None
+        self.lam = None
+
+    def _n(self, key):
+        return self.prefix + self.names[key]
+
+    def _widths(self):
+        return [("q", 2 * self.nh * self.dim), ("k", 2 * self.nkv * self.dim), ("v", self.nkv * self.vdim)]
+
+    def tensor_specs(self):
+        specs = {}
+        for k, n in self._widths():
+            specs[self._n(k)] = TensorSpec((n, self.hidden))
+            specs[self._n(k) + self.names["conv"]] = TensorSpec((n, self.taps), "filter")
+        for k in ("lq1", "lk1", "lq2", "lk2"):
+            specs[self._n(k)] = TensorSpec((self.dim,), "bias")
+        specs[self._n("o")] = TensorSpec((self.hidden, self.nh * self.vdim))
+        return specs
+
+    def _by_kv_head(self, rows):
+        """Query rows [heads, 2, dim, ...] in the order (kv head, map, head of the group, dim)."""
+        R = self.nh // self.nkv
+        t = rows.reshape(self.nkv, R, 2, self.dim, -1).permute(0, 2, 1, 3, 4)
+        return t.reshape(2 * self.nh * self.dim, -1)
+
+    def load(self, get):
+        q, qc = self._by_kv_head(get(self._n("q"))), self._by_kv_head(get(self._n("q") + self.names["conv"]))
+        self.w_in = _projection(torch.cat([q, get(self._n("k")), get(self._n("v"))], 0).contiguous())
+        self.conv = torch.cat([qc, get(self._n("k") + self.names["conv"]), get(self._n("v") + self.names["conv"])],
+                              0).float().contiguous()
+        self.w_o = _projection(get(self._n("o")))
+        l = {k: get(self._n(k)).double() for k in ("lq1", "lk1", "lq2", "lk2")}
+        # one number for the layer, made once from the stored vectors
+        self.lam = float(torch.exp((l["lq1"] * l["lk1"]).sum()) - torch.exp((l["lq2"] * l["lk2"]).sum())) + self.diff
+
+    def cache_need(self):
+        from .base import StateNeed
+        return (StateNeed((max(self.taps - 1, 0), self.channels)),
+                KvNeed(2 * self.nkv, self.dim, self.window, v_dim=self.vdim, v_heads=self.nkv))
+
+    def check(self, dtype):
+        if max(self.dim, self.vdim) > ops.WINDOW_ATTENTION_MAX_DIM:
+            raise ValueError(f"{self.prefix}: head sizes {self.dim} and {self.vdim} (at most {ops.WINDOW_ATTENTION_MAX_DIM})")
+        if not 1 <= self.taps <= ops.SHORT_CONV_MAX_TAPS:
+            raise ValueError(f"{self.prefix}: {self.taps} taps (at most {ops.SHORT_CONV_MAX_TAPS})")
+        cos, _ = self.position.tables("cpu")
+        if cos is not None and 2 * cos.shape[1] > self.dim:
+            raise ValueError(f"{self.prefix}: the rotation turns {2 * cos.shape[1]} values of maps of {self.dim}")
+
+    def forward(self, h, ctx, cache, owner=True):
+        N, act, dev = h.shape[0], h.dtype, h.device
+        conv_state, kv = cache
+        nq, nk = 2 * self.nh, 2 * self.nkv
+        cap = self.position.capacity
+        if cap is not None and ctx.max_position >= cap:
+            raise ValueError(f"position {ctx.max_position} is beyond the position encoding's capacity {cap}")
+        proj = linear(h, self.w_in, torch.float32)          # [N, q | k | v] float
+        mixed = torch.empty((N, self.channels), dtype=torch.float32, device=dev)
+        ops.short_conv(proj, self.conv, None, conv_state.state, ctx.tok_seq, ctx.tok_pos, ctx.seq_start, ctx.seq_past,
+                       ctx.seq_slot, mixed)
+        q = torch.empty((N, nq * self.dim), dtype=act, device=dev)
+        table = ctx.page_table(kv.group)
+        ops.window_intake(mixed, None, q, kv.k_pages, kv.v_pages, table, ctx.tok_seq, ctx.tok_pos, None, None, 0.0,
+                          nq, nk, self.dim, self.vdim, write_kv=owner, rotation=self.position.tables(dev), v_share=2)
+        maps = torch.empty((N, nq * self.vdim), dtype=act, device=dev)
+        if act == torch.bfloat16 and not ctx.one_token_each and ops.window_prefill_takes(self.dim, self.vdim):
+            ops.window_attention_prefill_bf16(q, kv.k_pages, kv.v_pages, table, ctx.seq_start, ctx.seq_past, maps,
+                                              self.scale, nq, nk, self.dim, self.vdim, window=self.window or 0, v_share=2)
+        else:
+            ops.window_attention(q, kv.k_pages, kv.v_pages, table, ctx.tok_seq, ctx.tok_pos, maps, self.scale, nq, nk,
+                                 self.dim, self.vdim, window=self.window or 0, v_share=2)
+        o = torch.empty((N, self.nh * self.vdim), dtype=act, device=dev)
+        ops.diff_heads(maps, o, self.lam, self.norm_eps, 1.0 - self.diff, self.nkv, self.nh // self.nkv, self.vdim)
+        return linear_for_sum(o, self.w_o)
+
+
 class ParallelMixers(Mixer):
     """Several mixers side by side that read the same input; the result is sum_i scale_i * mixer_i(h).  Each keeps
     what it needs for a sequence: the cache need is the tuple of theirs, and so is the cache view."""

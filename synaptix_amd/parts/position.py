@@ -118,3 +118,60 @@ class RotaryInterleaved(Position):
             cos, sin = self.host_tables()
             self._shared[key] = (torch.from_numpy(cos).to(device), torch.from_numpy(sin).to(device))
         return self._shared[key]
+
+
+class RotaryScaledHalfSplit(Position):
+    """The half-split rotation (value i < dims / 2 paired with value i + dims / 2, the rest passes) whose long waves are
+    stretched for contexts beyond the one the rates were made for.  With f_i = base^(-2i / dims) and, for a number of
+    turns t over the `original` context, place(t) = dims ln(original / (2 pi t)) / (2 ln base):
+
+        lo = max(floor(place(fast)), 0);  hi = min(ceil(place(slow)), dims - 1)
+        ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)
+        rate_i = f_i / factor * ramp_i + f_i * (1 - ramp_i)
+
+    and cos and sin both carry the factor 0.1 ln(factor) + 1.  factor None: the plain rates, no factor on cos and sin.
+    Angles are position * rate in 32-bit; tables [capacity, dims / 2], kept once for equal constants."""
+    capturable = True
+    _shared: dict = {}
+
+    def __init__(self, base: float, dims: int, capacity: int, factor: float | None = None, original: float | None = None,
+                 fast: float | None = None, slow: float | None = None):
+        if dims < 0 or dims % 2:
+            raise ValueError(f"rotated dims {dims} must be even and not negative")
+        if capacity <= 0:
+            raise ValueError("capacity must be positive")
+        if factor is not None and (original is None or fast is None or slow is None or not factor > 0.0):
+            raise ValueError("a scaled rotation needs factor, original, fast and slow")
+        self.base, self.dims, self.capacity = float(base), int(dims), int(capacity)
+        self.factor, self.original, self.fast, self.slow = factor, original, fast, slow
+
+    def rates(self):
+        """(rate_i as float64 [dims / 2], the factor on cos and sin)."""
+        import math
+        half = self.dims // 2
+        i = np.arange(half, dtype=np.float64)
+        f = np.power(np.float64(self.base), -2.0 * i / max(self.dims, 1))
+        if self.factor is None:
+            return f, 1.0
+
+        def place(turns):
+            return self.dims * math.log(self.original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.base))
+
+        lo, hi = max(math.floor(place(self.fast)), 0), min(math.ceil(place(self.slow)), self.dims - 1)
+        ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return f / self.factor * ramp + f * (1.0 - ramp), 0.1 * math.log(self.factor) + 1.0
+
+    def host_tables(self):
+        rates, mult = self.rates()
+        ang = np.arange(self.capacity, dtype=np.float32)[:, None] * rates.astype(np.float32)[None, :]
+        ang = ang.astype(np.float64)           # (the 32-bit angle itself, its cosine and sine taken exactly)
+        return (np.cos(ang) * mult).astype(np.float32), (np.sin(ang) * mult).astype(np.float32)
+
+    def tables(self, device):
+        if self.dims == 0:
+            return None, None
+        key = (self.base, self.dims, self.capacity, self.factor, self.original, self.fast, self.slow, str(device))
+        if key not in self._shared:
+            cos, sin = self.host_tables()
+            self._shared[key] = (torch.from_numpy(cos).to(device), torch.from_numpy(sin).to(device))
+        return self._shared[key]

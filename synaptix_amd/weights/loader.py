@@ -55,7 +55,8 @@ def check_source(specs: dict, source: WeightSource, ignored=(), where="") -> Non
     for n, spec in specs.items():
         if n in names:
             _, shape = source.info(n)
-            if tuple(shape) != tuple(spec.shape):
+            # (a size that a spec leaves open, None, is whatever the file holds)
+            if len(shape) != len(spec.shape) or any(w is not None and w != g for g, w in zip(shape, spec.shape)):
                 wrong.append((n, tuple(shape), tuple(spec.shape)))
     if missing or unexpected or wrong:
         raise WeightError(missing, unexpected, wrong, where)

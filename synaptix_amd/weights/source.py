@@ -17,7 +17,8 @@ from .safetensors_io import SafetensorsFile, resolve_shards, _NAMES
 class TensorSpec:
     """What a part expects under a name.  `kind` only matters to the random generator:
     "matrix" and "table" draw N(0, std), "gain" draws 1 + N(0, gain_std), "bias" N(0, gain_std), "positive"
-    |N(0, 1)| / 2 + 0.05, "mixing" (a square matrix) the identity + N(0, gain_std)."""
+    |N(0, 1)| / 2 + 0.05, "mixing" (a square matrix) the identity + N(0, gain_std), "filter" (the taps of short
+    convolutions) N(0, 1/2), "rate" (logarithms of decay rates) N(0, 1/2) - 1."""
     shape: tuple
     kind: str = "matrix"
 
@@ -112,12 +113,16 @@ class RandomSource(WeightSource):
         g = torch.Generator(device=self.device)
         g.manual_seed(tensor_seed(self.seed, name))
         shape = tuple(spec.shape)
+        if any(n is None for n in shape):
+            raise ValueError(f"tensor {name}: a size that only stored weights decide ({list(shape)}) cannot be drawn")
         if spec.kind == "gain":
             t = torch.randn(shape, generator=g, device=self.device, dtype=torch.float32) * self.gain_std + 1.0
         elif spec.kind == "bias":
             t = torch.randn(shape, generator=g, device=self.device, dtype=torch.float32) * self.gain_std
         elif spec.kind == "positive":
             t = torch.randn(shape, generator=g, device=self.device, dtype=torch.float32).abs() * 0.5 + 0.05
+        elif spec.kind in ("filter", "rate"):
+            t = torch.randn(shape, generator=g, device=self.device, dtype=torch.float32) * 0.5 - (1.0 if spec.kind == "rate" else 0.0)
         elif spec.kind == "mixing":
             t = (torch.randn(shape, generator=g, device=self.device, dtype=torch.float32) * self.gain_std
                  + torch.eye(shape[0], device=self.device))

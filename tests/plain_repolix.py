@@ -40,6 +40,22 @@ def short_conv(u, w, bias=None):
 
 
 # ---------------------------------------------------------------- mixer: state space with a scalar decay a head
+def state_space_cell(x, B, C, dt_raw, dt_bias, a_log, d_skip, S=None):
+    """x [T, H, P], B and C [T, G, N], dt_raw [T, H] -> y [T, H, P]; S [H, N, P] is updated in place if given."""
+    T, H, P = x.shape
+    G, N = B.shape[1], B.shape[2]
+    dt = softplus(dt_raw + dt_bias)
+    decay = torch.exp(-torch.exp(a_log) * dt)
+    S = torch.zeros(H, N, P, dtype=F64) if S is None else S
+    y = torch.zeros(T, H, P, dtype=F64)
+    for t in range(T):
+        for hd in range(H):
+            g = hd // (H // G)
+            S[hd] = decay[t, hd] * S[hd] + dt[t, hd] * torch.outer(B[t, g], x[t, hd])
+            y[t, hd] = S[hd].T @ C[t, g] + d_skip[hd] * x[t, hd]
+    return y
+
+
 def state_space(h, w, p, c, eps):
     T = h.shape[0]
     H, P, N, G = c["heads"], c["vdim"], c["state"], c["groups"]
@@ -50,15 +66,7 @@ def state_space(h, w, p, c, eps):
     x = xbc[:, :inner].view(T, H, P)
     B = xbc[:, inner:inner + G * N].view(T, G, N)
     C = xbc[:, inner + G * N:].view(T, G, N)
-    dt = softplus(dt + w[p + "dt_bias"])                                   # [T, H]
-    decay = torch.exp(-torch.exp(w[p + "A_log"]) * dt)
-    S = torch.zeros(H, N, P, dtype=F64)
-    y = torch.zeros(T, H, P, dtype=F64)
-    for t in range(T):
-        for hd in range(H):
-            g = hd // (H // G)
-            S[hd] = decay[t, hd] * S[hd] + dt[t, hd] * torch.outer(B[t, g], x[t, hd])
-            y[t, hd] = S[hd].T @ C[t, g] + w[p + "D"][hd] * x[t, hd]
+    y = state_space_cell(x, B, C, dt, w[p + "dt_bias"], w[p + "A_log"], w[p + "D"])
     y = y.reshape(T, inner) * silu(z)
     parts = c["norm_groups"]
     y = rms_norm(y.view(T, parts, inner // parts), None, eps).reshape(T, inner) * w[p + "norm"]
@@ -66,21 +74,19 @@ def state_space(h, w, p, c, eps):
 
 
 # ---------------------------------------------------------------- mixer: delta rule with a decay for every key channel
-def channel_delta(h, w, p, c, eps):
-    T = h.shape[0]
-    H, K, D, E = c["heads"], c["kv_heads"], c["dim"], c["vdim"]
+def delta_cell(q, k, v, beta_raw, a_raw, a_bias, a_log, S=None):
+    """q, k [T, K, D] (not yet unit vectors), v [T, H, E], beta_raw [T, H], a_raw [T, H, D], a_bias [H, D], a_log [H]
+    -> o [T, H, E]; S [H, D, E] is updated in place if given."""
+    T, K, D = q.shape
+    H, E = v.shape[1], v.shape[2]
 
     def unit(x):
         return x / torch.sqrt(x.pow(2).sum(-1, keepdim=True) + 1e-6)
 
-    q = silu(short_conv(h @ w[p + "q"].T, w[p + "q.conv"])).view(T, K, D)
-    k = silu(short_conv(h @ w[p + "k"].T, w[p + "k.conv"])).view(T, K, D)
-    v = silu(short_conv(h @ w[p + "v"].T, w[p + "v.conv"])).view(T, H, E)
     q, k = unit(q) * D ** -0.5, unit(k)
-    beta = torch.sigmoid(h @ w[p + "b"].T)                                     # [T, H]
-    a = (h @ w[p + "a1"].T) @ w[p + "a2"].T + w[p + "dt_bias"]
-    decay = torch.exp(-torch.exp(w[p + "A_log"])[None, :, None] * softplus(a).view(T, H, D))
-    S = torch.zeros(H, D, E, dtype=F64)
+    beta = torch.sigmoid(beta_raw)
+    decay = torch.exp(-torch.exp(a_log)[None, :, None] * softplus(a_raw + a_bias))
+    S = torch.zeros(H, D, E, dtype=F64) if S is None else S
     o = torch.zeros(T, H, E, dtype=F64)
     for t in range(T):
         for hd in range(H):
@@ -89,6 +95,17 @@ def channel_delta(h, w, p, c, eps):
             u = beta[t, hd] * (v[t, hd] - S[hd].T @ k[t, kv])
             S[hd] = S[hd] + torch.outer(k[t, kv], u)
             o[t, hd] = S[hd].T @ q[t, kv]
+    return o
+
+
+def channel_delta(h, w, p, c, eps):
+    T = h.shape[0]
+    H, K, D, E = c["heads"], c["kv_heads"], c["dim"], c["vdim"]
+    q = silu(short_conv(h @ w[p + "q"].T, w[p + "q.conv"])).view(T, K, D)
+    k = silu(short_conv(h @ w[p + "k"].T, w[p + "k.conv"])).view(T, K, D)
+    v = silu(short_conv(h @ w[p + "v"].T, w[p + "v.conv"])).view(T, H, E)
+    a = ((h @ w[p + "a1"].T) @ w[p + "a2"].T).view(T, H, D)
+    o = delta_cell(q, k, v, h @ w[p + "b"].T, a, w[p + "dt_bias"].view(H, D), w[p + "A_log"])
     o = rms_norm(o, w[p + "norm"], eps)
     gate = torch.sigmoid((h @ w[p + "g1"].T) @ w[p + "g2"].T).view(T, H, E)
     return (o * gate).reshape(T, H * E) @ w[p + "o"].T
@@ -138,6 +155,18 @@ def window_softmax(q, k, scale, window):
     return torch.softmax((scale * q @ k.T).masked_fill(~seen, -math.inf), -1)
 
 
+def two_maps(q, k, v, scale, window, lam, eps, post):
+    """q [T, H, 2, D], k [T, G, 2, D], v [T, G, E] -> [T, H, E]: rms_norm(a1 - lam a2) * post for each head."""
+    T, H, G, E = q.shape[0], q.shape[1], k.shape[1], v.shape[2]
+    o = torch.zeros(T, H, E, dtype=F64)
+    for hd in range(H):
+        g = hd // (H // G)
+        a1 = window_softmax(q[:, hd, 0], k[:, g, 0], scale, window) @ v[:, g]
+        a2 = window_softmax(q[:, hd, 1], k[:, g, 1], scale, window) @ v[:, g]
+        o[:, hd] = rms_norm(a1 - lam * a2, None, eps) * post
+    return o
+
+
 def differential_attention(h, w, p, c, eps, positions=None):
     T = h.shape[0]
     H, G, D, E = c["heads"], c["kv_heads"], c["dim"], c["vdim"]
@@ -148,12 +177,7 @@ def differential_attention(h, w, p, c, eps, positions=None):
     q, k = turn_halves(q, pos, c["rot"]), turn_halves(k, pos, c["rot"])
     lam = (torch.exp((w[p + "lq1"] * w[p + "lk1"]).sum()) - torch.exp((w[p + "lq2"] * w[p + "lk2"]).sum()) + c["diff"])
     window = (c.get("mask") or {}).get("size")
-    o = torch.zeros(T, H, E, dtype=F64)
-    for hd in range(H):
-        g = hd // (H // G)
-        a1 = window_softmax(q[:, hd, 0], k[:, g, 0], c["scale"], window) @ v[:, g]
-        a2 = window_softmax(q[:, hd, 1], k[:, g, 1], c["scale"], window) @ v[:, g]
-        o[:, hd] = rms_norm(a1 - lam * a2, None, eps) * (1.0 - c["diff"])
+    o = two_maps(q, k, v, c["scale"], window, lam, eps, 1.0 - c["diff"])
     return o.reshape(T, H * E) @ w[p + "o"].T
 
 
@@ -219,7 +243,7 @@ class PlainRepolix:
         """The residual after every layer [layers, T, W] and the logits [T, vocab] of one whole sequence."""
         c, w = self.c, self.w
         eps = c["norm"]["eps"]
-        x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)] * c["embedding"]["scale"]
+        x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)] * (c.get("embedding") or {}).get("scale", 1.0)
         after = []
         for i, layer in enumerate(c["layers"]):
             p = f"l{i}."

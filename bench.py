@@ -2,7 +2,7 @@
 """Throughput of the engine at a Qwen3 shape with random bf16 weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape 8b|4b|32b] [--batch 8] [--layers L]
-    python bench.py --design bizipel|kamivik [--sizes small,mid,large] [--prompt 2048] [--batch 8] [--window 1024]
+    python bench.py --design bizipel|kamivik|repolix [--sizes small,mid,large] [--prompt 2048] [--batch 8] [--window 1024]
 
 --shape 8b (the default) and 32b: a step is one decode step of `batch` sequences, each after a
 2,048-token prompt of uniform ids, run through the same captured graph and host loop that
@@ -28,6 +28,10 @@ weights), each with the time of every kernel entry point of one prompt step and 
 --design kamivik: the same for the Kamivik design: latent attention with a latent of 512 and a rotated part of 64 beside
 unrotated keys and values of the head size, every second layer with the window; a mixture of 8 x top experts of which each
 token uses `top`, top x the expert's width being the dense feed-forward's width.
+--design repolix: the same for the Repolix design: layers in the order state space (2 x width / 64 heads of 64 values, a
+state of 128 rows, 8 groups), delta rule (the heads and head size of the attention), attention in two maps of half the
+head size over shared values with the window, state space; gated experts of which each token uses top - 1 beside one
+shared expert (together the dense feed-forward's width), two identity experts, two groups of which one stays.
 
 Method after the reference's own harnesses (crates/synaptix-models/llm/qwen3/examples/format_perf.rs:41-122,
 crates/synaptix-cli/src/commands/bench.rs:35-96): synthetic ids, warm-up first, device synchronised
@@ -178,6 +182,14 @@ SIDE_BY_SIDE_SIZES = {     # layers, width, heads, kv heads, head size, feed-for
 
 
 KAMIVIK_EXPERTS = {"small": (4, 1024), "mid": (4, 2048), "large": (6, 2048)}      # (top, an expert's width); 8 x top experts
+REPOLIX_ORDER = ("mamba2", "channel_delta", "attention", "mamba2")
+
+
+def repolix_experts(size):
+    """(experts with matrices, identity experts, chosen a token, an expert's width): with the shared expert the active
+    width is the dense feed-forward's."""
+    top, eff = KAMIVIK_EXPERTS[size]
+    return 8 * (top - 1), 2, top - 1, eff
 
 
 def design_configs(design, size, window, context):
@@ -187,11 +199,25 @@ def design_configs(design, size, window, context):
     layers have latent attention (a latent of 512, 64 rotated values, unrotated keys and values of the head size; every
     second layer with the window) and a mixture of experts whose active width equals the dense feed-forward's."""
     from synaptix_amd import Qwen3Config
-    from synaptix_amd.config import BizipelConfig, KamivikConfig
+    from synaptix_amd.config import BizipelConfig, KamivikConfig, RepolixConfig
     L, W, nh, nkv, hd, ff, V = SIDE_BY_SIDE_SIZES[size]
     qwen = Qwen3Config.from_dict(dict(_COMMON, num_hidden_layers=L, hidden_size=W, num_attention_heads=nh,
                                       num_key_value_heads=nkv, head_dim=hd, intermediate_size=ff, vocab_size=V,
                                       tie_word_embeddings=design == "bizipel", max_position_embeddings=context))
+    if design == "repolix":
+        E, I, top, eff = repolix_experts(size)
+        mlp = {"kind": "moe", "expert": {"ff": eff, "limit": 7.0}, "shared": {"ff": eff, "limit": 7.0},
+               "router": {"experts": E, "identity": I, "top": top, "groups": {"count": 2, "keep": 1}}}
+        mixers = {"mamba2": {"heads": 2 * W // 64, "vdim": 64, "state": 128, "groups": 8, "norm_groups": 8, "conv": 4},
+                  "channel_delta": {"heads": nh, "kv_heads": nh, "dim": hd, "vdim": hd, "conv": 4},
+                  "attention": {"heads": nh, "kv_heads": nkv, "dim": hd // 2, "vdim": hd, "conv": 4, "diff": 0.5,
+                                "scale": (hd // 2) ** -0.5, "mask": {"size": window},
+                                "rot": {"base": 10000.0, "dims": hd // 2,
+                                        "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+        layers = [{"type": REPOLIX_ORDER[i % 4], "mixer": mixers[REPOLIX_ORDER[i % 4]], "mlp": mlp} for i in range(L)]
+        rep = RepolixConfig.from_dict({"architecture": "Repolix", "vocab": V, "width": W, "norm": {"eps": 1e-6},
+                                       "embedding": {"scale": float(W) ** 0.5}, "middle_rank": hd, "layers": layers})
+        return qwen, rep
     if design == "kamivik":
         top, eff = KAMIVIK_EXPERTS[size]
         layers = []
@@ -241,6 +267,12 @@ def designs_side_by_side(args) -> int:
                 top, eff = KAMIVIK_EXPERTS[size]
                 E, one = 8 * top, 2 * 2 * eff * cfg.width
                 touched = E * (1.0 - (1.0 - top / E) ** B)
+                weight_bytes -= int(len(cfg.layers) * (E - touched) * one)
+            if design == "repolix":
+                # likewise: the experts among the kept group's that B x top choices name (three matrices an expert)
+                E, I, top, eff = repolix_experts(size)
+                total, one = E + I, 3 * 2 * eff * cfg.width
+                touched = E * (1.0 - (1.0 - top / total) ** B)
                 weight_bytes -= int(len(cfg.layers) * (E - touched) * one)
             g = torch.Generator().manual_seed(0)
             prompt = torch.randint(0, cfg.vocab_size, (P,), generator=g).tolist()
@@ -312,7 +344,7 @@ def main() -> int:
                     help="the longest sequence (positions and cache a sequence; the contract's run has 8,192)")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
-    ap.add_argument("--design", default=None, choices=["bizipel", "kamivik"],
+    ap.add_argument("--design", default=None, choices=["bizipel", "kamivik", "repolix"],
                     help="another run than the default one: this design beside the Qwen3 decoder at equal layer sizes")
     ap.add_argument("--sizes", default="small,mid,large", help="with --design: which of small, mid, large")
     ap.add_argument("--window", type=int, default=1024, help="with --design: the keys a query of the new design sees")

@@ -26,8 +26,8 @@ def _rows(w):
     return w
 
 
-def embed(table, ids, resid):
-    resid.copy_(_rows(table)[ids.long()].to(F32))
+def embed(table, ids, resid, scale=1.0):
+    resid.copy_(_rows(table)[ids.long()].to(F32) * scale)
 
 
 def add_rmsnorm(resid, delta, gain, eps, out, rows=None, gain_offset=0.0):

@@ -142,7 +142,8 @@ def run_trace(folder: str, dtype: str, steps: list, max_tokens: int, out_dir: st
     done = [l for l in proc.stdout.splitlines() if l.startswith("done ")]
     assert done == [f"done {s['step']}" for s in steps], f"done lines: {done[:5]} ..."
     with open(os.path.join(folder, "config.json")) as f:
-        vocab = json.load(f)["vocab_size"]
+        cfg = json.load(f)
+    vocab = cfg["vocab_size"] if "vocab_size" in cfg else cfg["vocab"]
     out = {}
     for s in steps:
         p = os.path.join(out_dir, f"{s['step']}.f32")

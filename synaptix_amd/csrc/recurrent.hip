@@ -10,12 +10,12 @@
 //
 // Everything here is 32-bit FMA: inputs are the float sums of the projections, states are float.  The scans walk a
 // sequence's tokens in order; what runs side by side is (sequence, head, tile of 16 state columns): a wave holds 16
-// columns of a head's state in registers, four lanes a column, each with every fourth row.  A workgroup's waves (up to
-// four tiles of one head) share the token's vectors, which are staged through LDS sixteen tokens at a time.
+// columns of a head's state in registers, four lanes a column, each with a quarter of the rows.  A workgroup's waves (up
+// to four tiles of one head) share the token's vectors, which are staged through LDS sixteen tokens at a time.
 #include "common.h"
 
 #define RC_MAX_TAPS 16
-#define RC_TB 16            // tokens staged at a time
+#define RC_TB 32            // the most tokens staged at a time (fewer where LDS would not hold them)
 #define RC_ROWS_MAX 256     // rows of a head's state (N of the state space, key size of the delta rule)
 
 __device__ __forceinline__ float rc_silu(float z) { return z / (1.f + expf(-z)); }
@@ -88,31 +88,59 @@ SYN_EXPORT int syn_short_conv(const float* u, int u_stride, const float* w, cons
 }
 
 // ---------------------------------------------------------------- what the two scans share
-// lane = 16 * slice + column: the lane holds rows slice, slice + 4, ... of its column; R = rows / 4 rounded up
+// A wave holds 64 / SL columns of a head's state, SL lanes a column (SL = 4 or 16 slices), and a lane holds the rows
+// slice * R .. slice * R + R - 1 of its column (R = rows / SL rounded up to a multiple of 4; rows beyond the state's are
+// zeros that stay zeros).
+//   SL = 4:  lane = 16 * slice + column.  The state is read and written in pieces of 64 bytes: for single tokens, where
+//            the state is all that moves.
+//   SL = 16: lane = slice + 16 * column.  A token's chain of operations is a quarter as long, there are four times as many
+//            waves, and the sum over a column's slices stays inside a row of 16 lanes (four DPP additions, no trip through
+//            LDS): for prompts, whose tokens come one after another and wait for one another.
+// A token's vectors over the rows lie in LDS as SL pieces of R values, each followed by four unused ones, so that the
+// slices' 16-byte reads spread over the banks and no read needs a bound.
+#define RC_LD(R, SL) ((SL) * ((R) + 4))
+#define RC_LDS_BUDGET (60 * 1024)
+__device__ __forceinline__ int rc_at(int n, int R) { return (n / R) * (R + 4) + n % R; }
+template <int CTRL>
+__device__ __forceinline__ float rc_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+// the sum over the lanes that hold a column's slices, in all of them
+template <int SL>
 __device__ __forceinline__ float rc_sum_slices(float v) {
-  v += __shfl_xor(v, 16, SYN_WAVE);
-  v += __shfl_xor(v, 32, SYN_WAVE);
+  if constexpr (SL == 16) {
+    v += rc_dpp<0xB1>(v);       // lanes 1 0 3 2 of every four
+    v += rc_dpp<0x4E>(v);       // lanes 2 3 0 1
+    v += rc_dpp<0x141>(v);      // the other four of every eight (mirrored)
+    v += rc_dpp<0x140>(v);      // the other eight of the row (mirrored)
+  } else {
+#pragma unroll
+    for (int off = 64 / SL; off < SYN_WAVE; off <<= 1) v += __shfl_xor(v, off, SYN_WAVE);
+  }
   return v;
 }
+template <int SL> __device__ __forceinline__ int rc_slice(int lane) { return SL == 16 ? lane % 16 : lane / (64 / SL); }
+template <int SL> __device__ __forceinline__ int rc_col(int lane) { return SL == 16 ? lane / 16 : lane % (64 / SL); }
 
 // ---------------------------------------------------------------- state space with a scalar decay a head
 // xbc [N][inner + 2 G Ns] float: x (H x P), B (G x Ns), C (G x Ns) behind the convolution; dt: float rows of dt_stride
 // values, one a head, before bias and softplus; state [rows][H][Ns][P]; y [N][H * P] float (D x included).
-template <int R>
-__global__ void __launch_bounds__(256)
+template <int R, int SL>
+__global__ void __launch_bounds__(64 * SL)
 state_space_scan_kernel(const float* __restrict__ xbc, const float* __restrict__ dt, int dt_stride,
                         const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ d_skip,
                         float* __restrict__ state, int state_rows, const int* __restrict__ seq_start,
-                        const int* __restrict__ seq_slot, float* __restrict__ y, int H, int P, int Ns, int G) {
-  extern __shared__ float lds[];
-  float* Bs = lds;                          // [RC_TB][Ns]
-  float* Cs = Bs + RC_TB * Ns;              // [RC_TB][Ns]
-  float* xs = Cs + RC_TB * Ns;              // [RC_TB][64]   dt * x of the workgroup's columns
-  float* xr = xs + RC_TB * 64;              // [RC_TB][64]   x itself
-  float* dec = xr + RC_TB * 64;             // [RC_TB]
+                        const int* __restrict__ seq_slot, float* __restrict__ y, int H, int P, int Ns, int G, int tb_max) {
+  constexpr int LD = RC_LD(R, SL), COLS = 64 / SL;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* Bs = lds;                          // [tb_max][LD]
+  float* Cs = Bs + tb_max * LD;             // [tb_max][LD]
+  float* xs = Cs + tb_max * LD;             // [tb_max][64]   dt * x of the workgroup's columns
+  float* xr = xs + tb_max * 64;             // [tb_max][64]   x itself
+  float* dec = xr + tb_max * 64;            // [tb_max]
   const int head = blockIdx.x, b = blockIdx.y, p0 = blockIdx.z * 64;
-  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE, slice = lane / 16;
-  const int p = p0 + wave * 16 + lane % 16;
+  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE, slice = rc_slice<SL>(lane);
+  const int mine = wave * COLS + rc_col<SL>(lane), p = p0 + mine;       // this lane's column: of the workgroup's 64, of the head
   const bool col_ok = p < P;
   const int s0 = seq_start[b], n_new = seq_start[b + 1] - s0;
   int slot = seq_slot[b];
@@ -122,18 +150,19 @@ state_space_scan_kernel(const float* __restrict__ xbc, const float* __restrict__
   float s[R];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
-    const int n = slice + 4 * i;
+    const int n = slice * R + i;
     s[i] = (col_ok && n < Ns) ? S[(size_t)n * P + p] : 0.f;
   }
   const float A = -expf(a_log[head]), bias = dt_bias[head], D = d_skip[head];
-  for (int t0 = 0; t0 < n_new; t0 += RC_TB) {
-    const int tb = min(RC_TB, n_new - t0);
+  for (int t0 = 0; t0 < n_new; t0 += tb_max) {
+    const int tb = min(tb_max, n_new - t0);
     __syncthreads();
-    for (int e = tid; e < tb * Ns; e += blockDim.x) {
-      const int t = e / Ns, n = e % Ns;
+    for (int e = tid; e < tb * SL * R; e += blockDim.x) {
+      const int t = e / (SL * R), n = e % (SL * R);
       const float* row = xbc + (size_t)(s0 + t0 + t) * width + inner + grp * Ns;
-      Bs[e] = row[n];
-      Cs[e] = row[G * Ns + n];
+      const bool in = n < Ns;
+      Bs[t * LD + rc_at(n, R)] = in ? row[n] : 0.f;
+      Cs[t * LD + rc_at(n, R)] = in ? row[G * Ns + n] : 0.f;
     }
     for (int e = tid; e < tb * 64; e += blockDim.x) {
       const int t = e / 64, pp = p0 + e % 64;
@@ -145,48 +174,61 @@ state_space_scan_kernel(const float* __restrict__ xbc, const float* __restrict__
       if (e % 64 == 0) dec[t] = expf(A * step);
     }
     __syncthreads();
+#pragma unroll 4
     for (int t = 0; t < tb; ++t) {
-      const float a = dec[t], bx = xs[t * 64 + wave * 16 + lane % 16];
-      const float* Bt = Bs + t * Ns;
-      const float* Ct = Cs + t * Ns;
-      float acc = 0.f;
+      const float a = dec[t], bx = xs[t * 64 + mine];
+      const float4* Bt = (const float4*)(Bs + t * LD + slice * (R + 4));
+      const float4* Ct = (const float4*)(Cs + t * LD + slice * (R + 4));
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < R; ++i) {
-        const int n = slice + 4 * i;
-        if (n < Ns) {
-          s[i] = fmaf(a, s[i], bx * Bt[n]);
-          acc = fmaf(s[i], Ct[n], acc);
-        }
+      for (int i = 0; i < R; i += 4) {
+        const float4 bv = Bt[i / 4], cv = Ct[i / 4];
+        s[i] = fmaf(a, s[i], bx * bv.x), acc[0] = fmaf(s[i], cv.x, acc[0]);
+        s[i + 1] = fmaf(a, s[i + 1], bx * bv.y), acc[1] = fmaf(s[i + 1], cv.y, acc[1]);
+        s[i + 2] = fmaf(a, s[i + 2], bx * bv.z), acc[2] = fmaf(s[i + 2], cv.z, acc[2]);
+        s[i + 3] = fmaf(a, s[i + 3], bx * bv.w), acc[3] = fmaf(s[i + 3], cv.w, acc[3]);
       }
-      acc = rc_sum_slices(acc);
+      const float sum = rc_sum_slices<SL>((acc[0] + acc[1]) + (acc[2] + acc[3]));
       if (slice == 0 && col_ok)
-        y[(size_t)(s0 + t0 + t) * inner + head * P + p] = fmaf(D, xr[t * 64 + wave * 16 + lane % 16], acc);
+        y[(size_t)(s0 + t0 + t) * inner + head * P + p] = fmaf(D, xr[t * 64 + mine], sum);
     }
   }
 #pragma unroll
   for (int i = 0; i < R; ++i) {
-    const int n = slice + 4 * i;
+    const int n = slice * R + i;
     if (col_ok && n < Ns) S[(size_t)n * P + p] = s[i];
   }
 }
 
 SYN_EXPORT int syn_state_space_scan(const float* xbc, const float* dt, int dt_stride, const float* dt_bias,
                                     const float* a_log, const float* d_skip, float* state, int state_rows,
-                                    const int* seq_start, const int* seq_slot, int n_seqs, float* y, int H, int P, int Ns,
-                                    int G, hipStream_t stream) {
-  SYN_CHECK(n_seqs > 0 && H > 0 && P > 0 && Ns > 0 && G > 0, "state_space_scan: empty input");
+                                    const int* seq_start, const int* seq_slot, int n_seqs, int longest, float* y, int H,
+                                    int P, int Ns, int G, hipStream_t stream) {
+  SYN_CHECK(n_seqs > 0 && longest > 0 && H > 0 && P > 0 && Ns > 0 && G > 0, "state_space_scan: empty input");
   SYN_CHECK(H % G == 0, "state_space_scan: %d heads do not divide into %d groups", H, G);
   SYN_CHECK(Ns <= RC_ROWS_MAX, "state_space_scan: a state of %d rows (at most %d)", Ns, RC_ROWS_MAX);
   SYN_CHECK(dt_stride >= H && state_rows > 0, "state_space_scan: step rows of %d values for %d heads", dt_stride, H);
-  const int waves = min(4, (P + 15) / 16);
   const dim3 grid(H, n_seqs, (P + 63) / 64);
-  const size_t lds = (size_t)(2 * RC_TB * Ns + 2 * RC_TB * 64 + RC_TB) * sizeof(float);
-#define SYN_SS(R)                                                                                                     \
-  state_space_scan_kernel<R><<<grid, waves * SYN_WAVE, lds, stream>>>(xbc, dt, dt_stride, dt_bias, a_log, d_skip, state, \
-                                                                      state_rows, seq_start, seq_slot, y, H, P, Ns, G)
-  if (Ns <= 64) SYN_SS(16);
-  else if (Ns <= 128) SYN_SS(32);
-  else SYN_SS(64);
+  const int cols = min(P, 64);
+  // single tokens: four slices a wave (the state moves in pieces of 64 bytes); tokens in a row: sixteen
+#define SYN_SS(R, SL)                                                                                                   \
+  do {                                                                                                                  \
+    const int per_token = (2 * RC_LD(R, SL) + 2 * 64 + 1) * (int)sizeof(float);                                         \
+    const int tb = max(1, min(min(RC_TB, longest), RC_LDS_BUDGET / per_token));                                         \
+    const int waves = (cols + 64 / SL - 1) / (64 / SL);                                                                 \
+    state_space_scan_kernel<R, SL><<<grid, waves * SYN_WAVE, (size_t)tb * per_token, stream>>>(                         \
+        xbc, dt, dt_stride, dt_bias, a_log, d_skip, state, state_rows, seq_start, seq_slot, y, H, P, Ns, G, tb);        \
+  } while (0)
+  if (longest <= 1) {
+    if (Ns <= 32) SYN_SS(8, 4);
+    else if (Ns <= 64) SYN_SS(16, 4);
+    else if (Ns <= 128) SYN_SS(32, 4);
+    else SYN_SS(64, 4);
+  } else {
+    if (Ns <= 64) SYN_SS(4, 16);
+    else if (Ns <= 128) SYN_SS(8, 16);
+    else SYN_SS(16, 16);
+  }
 #undef SYN_SS
   SYN_LAUNCH_CHECK("state_space_scan");
   return 0;
@@ -194,26 +236,28 @@ SYN_EXPORT int syn_state_space_scan(const float* xbc, const float* dt, int dt_st
 
 // ---------------------------------------------------------------- delta rule with a decay for every key channel
 // qkv [N][(2 K + H E)] float behind the convolution: q (K heads x D), k (K x D), v (H x E); beta: float rows, one a head,
-// before the sigmoid; a: float rows of a_stride values, H * D of them used, before bias and softplus; state [rows][H][D][E]; o [N][H * E] float.
+// before the sigmoid; a: float rows of a_stride values, H * D of them used, before bias and softplus; state
+// [rows][H][D][E]; o [N][H * E] float.
 // Staged for each token: q and k as unit vectors (q also times q_scale), the decays, k . q.
-template <int R>
-__global__ void __launch_bounds__(256)
+template <int R, int SL>
+__global__ void __launch_bounds__(64 * SL)
 channel_delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ beta, int beta_stride,
                           const float* __restrict__ a, int a_stride, const float* __restrict__ a_bias,
-                          const float* __restrict__ a_log, float q_scale, float unit_eps, float* __restrict__ state, int state_rows,
-                          const int* __restrict__ seq_start, const int* __restrict__ seq_slot, float* __restrict__ o,
-                          int H, int K, int D, int E) {
-  extern __shared__ float lds[];
-  float* qs = lds;                          // [RC_TB][D]
-  float* ks = qs + RC_TB * D;               // [RC_TB][D]
-  float* gs = ks + RC_TB * D;               // [RC_TB][D]
-  float* vs = gs + RC_TB * D;               // [RC_TB][64]
-  float* kq = vs + RC_TB * 64;              // [RC_TB]
-  float* bt = kq + RC_TB;                   // [RC_TB]
+                          const float* __restrict__ a_log, float q_scale, float unit_eps, float* __restrict__ state,
+                          int state_rows, const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
+                          float* __restrict__ o, int H, int K, int D, int E, int tb_max) {
+  constexpr int LD = RC_LD(R, SL), COLS = 64 / SL;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* qs = lds;                          // [tb_max][LD]
+  float* ks = qs + tb_max * LD;             // [tb_max][LD]
+  float* gs = ks + tb_max * LD;             // [tb_max][LD]
+  float* vs = gs + tb_max * LD;             // [tb_max][64]
+  float* kq = vs + tb_max * 64;             // [tb_max]
+  float* bt = kq + tb_max;                  // [tb_max]
   const int head = blockIdx.x, b = blockIdx.y, p0 = blockIdx.z * 64;
-  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE, slice = lane / 16;
+  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE, slice = rc_slice<SL>(lane);
   const int n_waves = blockDim.x / SYN_WAVE;
-  const int p = p0 + wave * 16 + lane % 16;
+  const int mine = wave * COLS + rc_col<SL>(lane), p = p0 + mine;
   const bool col_ok = p < E;
   const int s0 = seq_start[b], n_new = seq_start[b + 1] - s0;
   int slot = seq_slot[b];
@@ -223,12 +267,12 @@ channel_delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict
   float s[R];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
-    const int n = slice + 4 * i;
+    const int n = slice * R + i;
     s[i] = (col_ok && n < D) ? S[(size_t)n * E + p] : 0.f;
   }
   const float A = -expf(a_log[head]);
-  for (int t0 = 0; t0 < n_new; t0 += RC_TB) {
-    const int tb = min(RC_TB, n_new - t0);
+  for (int t0 = 0; t0 < n_new; t0 += tb_max) {
+    const int tb = min(tb_max, n_new - t0);
     __syncthreads();
     for (int t = wave; t < tb; t += n_waves) {
       const size_t tok = s0 + t0 + t;
@@ -241,10 +285,12 @@ channel_delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict
       }
       sq = wave_sum(sq), sk = wave_sum(sk), dot = wave_sum(dot);
       const float iq = q_scale / sqrtf(sq + unit_eps), ik = 1.f / sqrtf(sk + unit_eps);
-      for (int d = lane; d < D; d += SYN_WAVE) {
-        qs[t * D + d] = qr[d] * iq;
-        ks[t * D + d] = kr[d] * ik;
-        gs[t * D + d] = expf(A * rc_softplus(a[tok * (size_t)a_stride + head * D + d] + a_bias[head * D + d]));
+      for (int d = lane; d < SL * R; d += SYN_WAVE) {      // (rows beyond the keys: zeros, and a decay of one)
+        const bool in = d < D;
+        const int at = t * LD + rc_at(d, R);
+        qs[at] = in ? qr[d] * iq : 0.f;
+        ks[at] = in ? kr[d] * ik : 0.f;
+        gs[at] = in ? expf(A * rc_softplus(a[tok * (size_t)a_stride + head * D + d] + a_bias[head * D + d])) : 1.f;
       }
       if (lane == 0) {
         kq[t] = dot * iq * ik;
@@ -256,57 +302,70 @@ channel_delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict
       }
     }
     __syncthreads();
+#pragma unroll 2
     for (int t = 0; t < tb; ++t) {
-      const float* qt = qs + t * D;
-      const float* kt = ks + t * D;
-      const float* gt = gs + t * D;
-      float rk = 0.f, rq = 0.f;
+      const float4* qt = (const float4*)(qs + t * LD + slice * (R + 4));
+      const float4* kt = (const float4*)(ks + t * LD + slice * (R + 4));
+      const float4* gt = (const float4*)(gs + t * LD + slice * (R + 4));
+      float rk[4] = {0.f, 0.f, 0.f, 0.f}, rq[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < R; ++i) {
-        const int n = slice + 4 * i;
-        if (n < D) {
-          s[i] *= gt[n];
-          rk = fmaf(s[i], kt[n], rk);
-          rq = fmaf(s[i], qt[n], rq);
-        }
+      for (int i = 0; i < R; i += 4) {
+        const float4 gv = gt[i / 4], kv = kt[i / 4], qv = qt[i / 4];
+        s[i] *= gv.x, rk[0] = fmaf(s[i], kv.x, rk[0]), rq[0] = fmaf(s[i], qv.x, rq[0]);
+        s[i + 1] *= gv.y, rk[1] = fmaf(s[i + 1], kv.y, rk[1]), rq[1] = fmaf(s[i + 1], qv.y, rq[1]);
+        s[i + 2] *= gv.z, rk[2] = fmaf(s[i + 2], kv.z, rk[2]), rq[2] = fmaf(s[i + 2], qv.z, rq[2]);
+        s[i + 3] *= gv.w, rk[3] = fmaf(s[i + 3], kv.w, rk[3]), rq[3] = fmaf(s[i + 3], qv.w, rq[3]);
       }
-      rk = rc_sum_slices(rk), rq = rc_sum_slices(rq);
-      const float u = bt[t] * (vs[t * 64 + wave * 16 + lane % 16] - rk);
+      const float rks = rc_sum_slices<SL>((rk[0] + rk[1]) + (rk[2] + rk[3]));
+      const float rqs = rc_sum_slices<SL>((rq[0] + rq[1]) + (rq[2] + rq[3]));
+      const float u = bt[t] * (vs[t * 64 + mine] - rks);
 #pragma unroll
-      for (int i = 0; i < R; ++i) {
-        const int n = slice + 4 * i;
-        if (n < D) s[i] = fmaf(kt[n], u, s[i]);
+      for (int i = 0; i < R; i += 4) {
+        const float4 kv = kt[i / 4];
+        s[i] = fmaf(kv.x, u, s[i]), s[i + 1] = fmaf(kv.y, u, s[i + 1]);
+        s[i + 2] = fmaf(kv.z, u, s[i + 2]), s[i + 3] = fmaf(kv.w, u, s[i + 3]);
       }
       // the read-out sees this token's write: (S + k u^T)^T q = S^T q + u (k . q)
-      if (slice == 0 && col_ok) o[(size_t)(s0 + t0 + t) * H * E + head * E + p] = fmaf(u, kq[t], rq);
+      if (slice == 0 && col_ok) o[(size_t)(s0 + t0 + t) * H * E + head * E + p] = fmaf(u, kq[t], rqs);
     }
   }
 #pragma unroll
   for (int i = 0; i < R; ++i) {
-    const int n = slice + 4 * i;
+    const int n = slice * R + i;
     if (col_ok && n < D) S[(size_t)n * E + p] = s[i];
   }
 }
 
 SYN_EXPORT int syn_channel_delta_scan(const float* qkv, const float* beta, int beta_stride, const float* a, int a_stride,
                                       const float* a_bias, const float* a_log, float q_scale, float unit_eps, float* state,
-                                      int state_rows, const int* seq_start, const int* seq_slot, int n_seqs, float* o, int H,
-                                      int K, int D, int E, hipStream_t stream) {
-  SYN_CHECK(n_seqs > 0 && H > 0 && K > 0 && D > 0 && E > 0, "channel_delta_scan: empty input");
+                                      int state_rows, const int* seq_start, const int* seq_slot, int n_seqs, int longest,
+                                      float* o, int H, int K, int D, int E, hipStream_t stream) {
+  SYN_CHECK(n_seqs > 0 && longest > 0 && H > 0 && K > 0 && D > 0 && E > 0, "channel_delta_scan: empty input");
   SYN_CHECK(H % K == 0, "channel_delta_scan: %d heads do not divide into %d key heads", H, K);
   SYN_CHECK(D <= RC_ROWS_MAX, "channel_delta_scan: keys of %d values (at most %d)", D, RC_ROWS_MAX);
   SYN_CHECK(beta_stride >= H && state_rows > 0, "channel_delta_scan: rows of %d values for %d heads", beta_stride, H);
   SYN_CHECK(a_stride >= H * D, "channel_delta_scan: decay rows of %d values for %d heads of %d", a_stride, H, D);
-  const int waves = min(4, (E + 15) / 16);
   const dim3 grid(H, n_seqs, (E + 63) / 64);
-  const size_t lds = (size_t)(3 * RC_TB * D + RC_TB * 64 + 2 * RC_TB) * sizeof(float);
-#define SYN_CD(R)                                                                                                       \
-  channel_delta_scan_kernel<R><<<grid, waves * SYN_WAVE, lds, stream>>>(qkv, beta, beta_stride, a, a_stride, a_bias, a_log, q_scale, \
-                                                                        unit_eps, state, state_rows, seq_start, seq_slot, \
-                                                                        o, H, K, D, E)
-  if (D <= 64) SYN_CD(16);
-  else if (D <= 128) SYN_CD(32);
-  else SYN_CD(64);
+  const int cols = min(E, 64);
+#define SYN_CD(R, SL)                                                                                                   \
+  do {                                                                                                                  \
+    const int per_token = (3 * RC_LD(R, SL) + 64 + 2) * (int)sizeof(float);                                             \
+    const int tb = max(1, min(min(RC_TB, longest), RC_LDS_BUDGET / per_token));                                         \
+    const int waves = (cols + 64 / SL - 1) / (64 / SL);                                                                 \
+    channel_delta_scan_kernel<R, SL><<<grid, waves * SYN_WAVE, (size_t)tb * per_token, stream>>>(                       \
+        qkv, beta, beta_stride, a, a_stride, a_bias, a_log, q_scale, unit_eps, state, state_rows, seq_start, seq_slot,  \
+        o, H, K, D, E, tb);                                                                                             \
+  } while (0)
+  if (longest <= 1) {
+    if (D <= 32) SYN_CD(8, 4);
+    else if (D <= 64) SYN_CD(16, 4);
+    else if (D <= 128) SYN_CD(32, 4);
+    else SYN_CD(64, 4);
+  } else {
+    if (D <= 64) SYN_CD(4, 16);
+    else if (D <= 128) SYN_CD(8, 16);
+    else SYN_CD(16, 16);
+  }
 #undef SYN_CD
   SYN_LAUNCH_CHECK("channel_delta_scan");
   return 0;

@@ -1061,11 +1061,14 @@ def short_conv(u, weight, bias, state, tok_seq, tok_pos, seq_start, seq_past, se
           taps, _stream())
 
 
-def state_space_scan(xbc, dt, dt_bias, a_log, d_skip, state, seq_start, seq_slot, out, n_heads, vdim, n_state, n_groups):
+def state_space_scan(xbc, dt, dt_bias, a_log, d_skip, state, seq_start, seq_slot, out, n_heads, vdim, n_state, n_groups,
+                     single_tokens=False):
     """The state space with a scalar decay a head over the new tokens of every sequence of the step, in order:
         step = softplus(dt + dt_bias[h]);  S <- exp(-exp(a_log[h]) step) S + step B x^T;  y = S^T C + d_skip[h] x
     xbc float [N, H * vdim + 2 G * n_state]: x, B and C (head h reads group h // (H / G)); dt a float view [N, >= H];
-    state float [rows, H, n_state, vdim] (row seq_slot[b]; a negative slot: the last row); out float [N, H * vdim]."""
+    state float [rows, H, n_state, vdim] (row seq_slot[b]; a negative slot: the last row); out float [N, H * vdim].
+    single_tokens: every sequence brings one token (the kernel is then laid out for moving the state, not for a chain of
+    tokens; the results are the same)."""
     H, G = n_heads, n_groups
     if G <= 0 or H % G:
         raise KernelError(f"state_space_scan: {H} heads do not divide into {G} groups")
@@ -1080,19 +1083,20 @@ def state_space_scan(xbc, dt, dt_bias, a_log, d_skip, state, seq_start, seq_slot
     B = _step_seqs("state_space_scan", seq_start, seq_slot)
     _need(out, "state_space_scan.out", _F32, (N, H * vdim))
     _call(load_library("core"), "syn_state_space_scan", _ptr(xbc), _ptr(dt), stride, _ptr(dt_bias), _ptr(a_log),
-          _ptr(d_skip), _ptr(state), state.shape[0], _ptr(seq_start), _ptr(seq_slot), B, _ptr(out), H, vdim, n_state, G,
-          _stream())
+          _ptr(d_skip), _ptr(state), state.shape[0], _ptr(seq_start), _ptr(seq_slot), B, 1 if single_tokens else max(N, 2),
+          _ptr(out), H, vdim, n_state, G, _stream())
 
 
 def channel_delta_scan(qkv, beta, a, a_bias, a_log, q_scale, unit_eps, state, seq_start, seq_slot, out, n_heads,
-                       n_key_heads, dim, vdim):
+                       n_key_heads, dim, vdim, single_tokens=False):
     """The delta rule with a decay for every key channel over the new tokens of every sequence of the step, in order.
     With q and k made unit vectors (x / sqrt(sum x^2 + unit_eps); q also times q_scale), b = sigmoid(beta) and
     g = exp(-exp(a_log[h]) softplus(a + a_bias)) for each (head, key channel):
         S <- diag(g) S;  u = b (v - S^T k);  S <- S + k u^T;  o = S^T q
     qkv float [N, 2 K * dim + H * vdim]: q and k of the K key heads (head h reads key head h // (H / K)), v; beta a
     float view [N, >= H]; a a float view [N, >= H * dim]; a_bias float [H * dim]; a_log float [H]; state float
-    [rows, H, dim, vdim] (row seq_slot[b]; a negative slot: the last row); out float [N, H * vdim]."""
+    [rows, H, dim, vdim] (row seq_slot[b]; a negative slot: the last row); out float [N, H * vdim].
+    single_tokens: as for state_space_scan."""
     H, K = n_heads, n_key_heads
     if K <= 0 or H % K:
         raise KernelError(f"channel_delta_scan: {H} heads do not divide into {K} key heads")
@@ -1110,7 +1114,7 @@ def channel_delta_scan(qkv, beta, a, a_bias, a_log, q_scale, unit_eps, state, se
     _call(load_library("core"), "syn_channel_delta_scan", _ptr(qkv), _ptr(beta), stride, _ptr(a), a_stride, _ptr(a_bias),
           _ptr(a_log),
           ctypes.c_float(q_scale), ctypes.c_float(unit_eps), _ptr(state), state.shape[0], _ptr(seq_start), _ptr(seq_slot), B,
-          _ptr(out), H, K, dim, vdim, _stream())
+          1 if single_tokens else max(N, 2), _ptr(out), H, K, dim, vdim, _stream())
 
 
 def diff_heads(a, out, lam, eps, post, n_kv_heads, heads_per_kv, vdim):

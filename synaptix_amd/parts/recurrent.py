@@ -88,7 +88,8 @@ class StateSpaceMixer(Mixer):
                        ctx.tok_pos, ctx.seq_start, ctx.seq_past, ctx.seq_slot, xbc, silu=True)
         y = torch.empty((N, inner), dtype=torch.float32, device=h.device)
         ops.state_space_scan(xbc, proj[:, inner + self.channels:], self.dt_bias, self.a_log, self.d, cell.state,
-                             ctx.seq_start, ctx.seq_slot, y, self.nh, self.vdim, self.ns, self.ng)
+                             ctx.seq_start, ctx.seq_slot, y, self.nh, self.vdim, self.ns, self.ng,
+                             single_tokens=ctx.one_token_each)
         o = torch.empty((N, inner), dtype=h.dtype, device=h.device)
         ops.head_norm_gate(y, self.gain, self.norm_eps, proj[:, :inner], o, self.norm_groups, inner // self.norm_groups,
                            silu_first=True)
@@ -183,7 +184,8 @@ class ChannelDeltaMixer(Mixer):
                        ctx.seq_past, ctx.seq_slot, qkv, silu=True)
         raw = torch.empty((N, H * self.vdim), dtype=torch.float32, device=h.device)
         ops.channel_delta_scan(qkv, proj[:, self.channels:], wide[:, :H * self.dim], self.a_bias, self.a_log, self.q_scale, self.UNIT_EPS,
-                               cell.state, ctx.seq_start, ctx.seq_slot, raw, H, self.nk, self.dim, self.vdim)
+                               cell.state, ctx.seq_start, ctx.seq_slot, raw, H, self.nk, self.dim, self.vdim,
+                               single_tokens=ctx.one_token_each)
         o = torch.empty((N, H * self.vdim), dtype=h.dtype, device=h.device)
         ops.head_norm_gate(raw, self.gain, self.norm_eps, wide[:, H * self.dim:], o, H, self.vdim)
         return linear_for_sum(o, self.w_o)

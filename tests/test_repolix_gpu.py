@@ -130,7 +130,7 @@ def test_state_space_scan_keeps_far_tokens(H, Pv, G, N):
         wide[:, 9:] = dev(dts)
         out = torch.empty((st.N, H * Pv), dtype=torch.float32, device=DEV)
         ops.state_space_scan(dev(xbc), wide[:, 9:], dev(bias), dev(a_log), dev(d), state, st.seq_start, st.seq_slot, out,
-                             H, Pv, N, G)
+                             H, Pv, N, G, single_tokens=all(n == 1 for n in portion))
         for i, n in enumerate(portion):
             got[i].append(out[st.starts[i]:st.starts[i + 1]].cpu().double().view(n, H, Pv))
             fed[i] += n
@@ -168,7 +168,8 @@ def test_channel_delta_scan(H, K, D, E):
         wide[:, 3 + H:3 + H + H * D] = dev(torch.cat(cut(4)))
         out = torch.empty((st.N, H * E), dtype=torch.float32, device=DEV)
         ops.channel_delta_scan(dev(qkv), wide[:, 3:3 + H], wide[:, 3 + H:3 + H + H * D], dev(a_bias.reshape(-1)), dev(a_log),
-                               D ** -0.5, 1e-6, state, st.seq_start, st.seq_slot, out, H, K, D, E)
+                               D ** -0.5, 1e-6, state, st.seq_start, st.seq_slot, out, H, K, D, E,
+                               single_tokens=all(n == 1 for n in portion))
         for i, n in enumerate(portion):
             got[i].append(out[st.starts[i]:st.starts[i + 1]].cpu().double().view(n, H, E))
             fed[i] += n

@@ -8,7 +8,8 @@
 //   * every group takes all M rows (a linear map for each head of a token): A, W and out move on by a fixed
 //     number of elements from one group to the next.
 // Epilogue, in this order and each optional: the exact GELU 0.5 z (1 + erf(z / sqrt 2)); a weight of the row;
-// sigmoid of a gate value read from float rows.  Sums are 32-bit.  bf16 operands whose K is a multiple of 32 run on
+// sigmoid of a gate value read from float rows.  Or, with `pair`: W's rows come in pairs (2 j: the gate row of output j,
+// 2 j + 1: its up row) and what is stored is the gated activation of the two sums (gated, csrc/common.h), N / 2 columns.  Sums are 32-bit.  bf16 operands whose K is a multiple of 32 run on
 // the matrix cores: with few rows a group 16x16x32 with operands straight from memory as 16-byte pieces of rows (no
 // LDS: a wave computes 32 rows x 64 columns), with many rows tiles of 128 x 128 through LDS (any K that is a multiple
 // of 8); everything else, and all of the 32-bit path, is plain FMA with one wave a (row, 8 columns).
@@ -33,6 +34,8 @@ struct GroupedArgs {
   long gate_ld, gate_group;
   int gate_col;
   int act;                  // 0: none, 1: exact GELU
+  int pair;                 // 0: none; else 1 + the code of the gated activation over pairs of rows of W
+  float limit;              // that activation's bound, if it has one
   int M, N, K, groups;
   int w_packed;             // W[group] lies in the order of the fragments: [N / 16][K / 32][64 lanes][8] with
                             // lane = 16 (k % 32 / 8) + n % 16 (bf16, N a multiple of 16, K of 32); 0: plain rows
@@ -52,6 +55,13 @@ __device__ __forceinline__ float grouped_epilogue(const GroupedArgs& g, float v,
     const float z = g.gate[(size_t)r * g.gate_ld + (size_t)b * g.gate_group + (size_t)n * g.gate_col];
     v *= 1.f / (1.f + expf(-z));
   }
+  return v;
+}
+
+// the pair (gate sum, up sum) of output column n / 2 (n even)
+__device__ __forceinline__ float grouped_pair(const GroupedArgs& g, float gate, float up, int r) {
+  float v = gated(g.pair - 1, gate, up, g.limit);
+  if (g.row_weight) v *= g.row_weight[r];
   return v;
 }
 
@@ -89,6 +99,14 @@ __global__ void __launch_bounds__(256) grouped_product_simt_kernel(GroupedArgs g
     for (int c = 0; c < 8; ++c)
       if (n0 + c < g.N)
         acc[c] = fmaf(x, to_f32<T>(w[g.w_packed ? packed_at(n0 + c, k, g.K / 32) : (size_t)(n0 + c) * g.ldw + k]), acc[c]);
+  }
+  if (g.pair) {
+#pragma unroll
+    for (int c = 0; c < 8; c += 2) {
+      const float gate = wave_sum(acc[c]), up = wave_sum(acc[c + 1]);
+      if (lane == 0 && n0 + c < g.N) grouped_store(g, r, b, (n0 + c) / 2, grouped_pair(g, gate, up, r));
+    }
+    return;
   }
 #pragma unroll
   for (int c = 0; c < 8; ++c) {
@@ -202,7 +220,11 @@ __global__ void __launch_bounds__(256) grouped_product_mfma_kernel(GroupedArgs g
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int n = n0 + nb * 16 + q * 4 + e;
-        if (n < g.N) grouped_store(g, r, b, n, grouped_epilogue(g, acc[mb][nb][e], r, b, n));
+        if (g.pair) {      // (a lane holds four consecutive outputs: two pairs)
+          if (e % 2 == 0 && n < g.N) grouped_store(g, r, b, n / 2, grouped_pair(g, acc[mb][nb][e], acc[mb][nb][e + (e % 2 == 0)], r));
+        } else if (n < g.N) {
+          grouped_store(g, r, b, n, grouped_epilogue(g, acc[mb][nb][e], r, b, n));
+        }
       }
   }
 }
@@ -325,7 +347,12 @@ __global__ void __launch_bounds__(256) grouped_product_tiled_kernel(GroupedArgs 
       for (int e = 0; e < 16; ++e) {
         const int r = row0 + wm + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
         const int n = n0 + wn + j * 32 + lane % 32;
-        if (r < row_end && n < g.N) grouped_store(g, r, b, n, grouped_epilogue(g, acc[i][j][e], r, b, n));
+        if (g.pair) {      // (neighbouring lanes hold neighbouring outputs: the even lane takes its neighbour's up sum)
+          const float up = __shfl_xor(acc[i][j][e], 1, SYN_WAVE);
+          if (lane % 2 == 0 && r < row_end && n < g.N) grouped_store(g, r, b, n / 2, grouped_pair(g, acc[i][j][e], up, r));
+        } else if (r < row_end && n < g.N) {
+          grouped_store(g, r, b, n, grouped_epilogue(g, acc[i][j][e], r, b, n));
+        }
       }
 }
 
@@ -334,9 +361,12 @@ SYN_EXPORT int syn_grouped_product(const void* a, long lda, long a_group, const 
                                    long ldo, long o_group, int in_is_f32, int out_is_f32, const int* seg_start,
                                    const int* a_rows, const int* o_rows, const float* row_weight, const float* gate,
                                    long gate_ld, long gate_group, int gate_col, int act, int M, int N, int K, int groups,
-                                   int rows_bound, int force_simt, int w_packed, hipStream_t stream) {
+                                   int rows_bound, int force_simt, int w_packed, int pair, float limit,
+                                   hipStream_t stream) {
   SYN_CHECK(M > 0 && N > 0 && K > 0 && groups > 0, "grouped_product: empty input (%d rows, %d x %d, %d groups)", M, N, K, groups);
   SYN_CHECK(act == 0 || act == 1, "grouped_product: unknown activation code %d", act);
+  SYN_CHECK(pair >= 0 && pair <= SYN_ACT_COUNT && (pair == 0 || (N % 2 == 0 && act == 0 && gate == nullptr)),
+            "grouped_product: a gated activation (code %d) over %d rows of W in pairs, with no other activation", pair - 1, N);
   SYN_CHECK(seg_start != nullptr || (a_rows == nullptr && o_rows == nullptr && row_weight == nullptr),
             "grouped_product: index lists and row weights come with segments");
   SYN_CHECK(seg_start == nullptr || rows_bound > 0, "grouped_product: segments over %d rows", rows_bound);
@@ -344,7 +374,7 @@ SYN_EXPORT int syn_grouped_product(const void* a, long lda, long a_group, const 
   SYN_CHECK(!w_packed || (!in_is_f32 && N % 16 == 0 && K % 32 == 0),
             "grouped_product: matrices in fragment order are bf16 of %d x %d (multiples of 16 and 32)?", N, K);
   const GroupedArgs g = {a, lda, a_group, w, w_group, ldw, out, ldo, o_group, out_is_f32, seg_start, a_rows, o_rows,
-                         row_weight, gate, gate_ld, gate_group, gate_col, act, M, N, K, groups, w_packed};
+                         row_weight, gate, gate_ld, gate_group, gate_col, act, pair, limit, M, N, K, groups, w_packed};
   const bool aligned = K % 32 == 0 && lda % 8 == 0 && a_group % 8 == 0 && ldw % 8 == 0 && w_group % 8 == 0 &&
                        (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0;
   // many rows a group (on average, where the host does not know the segments): the tiles through LDS

@@ -70,6 +70,34 @@ short_conv_state_kernel(const float* __restrict__ u, int u_stride, float* __rest
     if (i < keep) st[(size_t)i * C + c] = v[i];
 }
 
+// Single tokens (every sequence of the step brings one): output and the state's shift in one pass, one thread a
+// (sequence, channel), which reads what it needs before it writes.
+__global__ void __launch_bounds__(256)
+short_conv_single_kernel(const float* __restrict__ u, int u_stride, const float* __restrict__ w, const float* __restrict__ bias,
+                         int act, float* __restrict__ state, int state_rows, const int* __restrict__ seq_start,
+                         const int* __restrict__ seq_slot, float* __restrict__ out, int C, int taps) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x, b = blockIdx.x;
+  if (c >= C) return;
+  int slot = seq_slot[b];
+  if (slot < 0 || slot >= state_rows) slot = state_rows - 1;
+  const int n = seq_start[b], keep = taps - 1;
+  float* st = state + (size_t)slot * keep * C;
+  const float now = u[(size_t)n * u_stride + c];
+  float v[RC_MAX_TAPS];
+  float acc = bias ? bias[c] : 0.f;
+#pragma unroll
+  for (int i = 0; i < RC_MAX_TAPS; ++i)
+    if (i < keep) {
+      v[i] = st[(size_t)i * C + c];
+      acc = fmaf(w[(size_t)c * taps + i], v[i], acc);
+    }
+  acc = fmaf(w[(size_t)c * taps + keep], now, acc);
+  out[(size_t)n * C + c] = act ? rc_silu(acc) : acc;
+#pragma unroll
+  for (int i = 0; i < RC_MAX_TAPS; ++i)
+    if (i < keep) st[(size_t)i * C + c] = i + 1 < keep ? v[i + 1 < RC_MAX_TAPS ? i + 1 : i] : now;
+}
+
 SYN_EXPORT int syn_short_conv(const float* u, int u_stride, const float* w, const float* bias, int act, float* state,
                               int state_rows, const int* tok_seq, const int* tok_pos, const int* seq_start,
                               const int* seq_past, const int* seq_slot, float* out, int n_tokens, int n_seqs, int C,
@@ -78,6 +106,12 @@ SYN_EXPORT int syn_short_conv(const float* u, int u_stride, const float* w, cons
   SYN_CHECK(taps >= 1 && taps <= RC_MAX_TAPS, "short_conv: %d taps (1 to %d)", taps, RC_MAX_TAPS);
   SYN_CHECK(u_stride >= C && state_rows > 0, "short_conv: rows of %d values for %d channels", u_stride, C);
   const int bx = (C + 255) / 256;
+  if (n_tokens == n_seqs) {      // (a step brings at least one token for each of its sequences: here exactly one)
+    short_conv_single_kernel<<<dim3(n_seqs, bx), 256, 0, stream>>>(u, u_stride, w, bias, act, state, state_rows, seq_start,
+                                                                  seq_slot, out, C, taps);
+    SYN_LAUNCH_CHECK("short_conv_single");
+    return 0;
+  }
   short_conv_kernel<<<dim3(n_tokens, bx), 256, 0, stream>>>(u, u_stride, w, bias, act, state, state_rows, tok_seq, tok_pos,
                                                            seq_past, seq_slot, out, n_tokens, C, taps);
   SYN_LAUNCH_CHECK("short_conv");

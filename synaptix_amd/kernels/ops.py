@@ -1041,7 +1041,8 @@ def short_conv(u, weight, bias, state, tok_seq, tok_pos, seq_start, seq_past, se
     u: a float view [N, C] whose rows may be pieces of longer rows (columns of a fused projection); weight float
     [C, taps]; bias float [C] or None; state float [rows, taps - 1, C]: the last taps - 1 inputs of the sequence in row
     seq_slot[b] (a negative slot: the last row), read for the tokens before this step and written for the next one;
-    out float [N, C]."""
+    out float [N, C].  Every sequence of the step brings at least one token (with as many tokens as sequences, one each:
+    output and state then take one launch)."""
     _need(weight, "short_conv.weight", _F32, (None, None))
     C, taps = weight.shape
     N = tok_seq.shape[0]
@@ -1240,12 +1241,13 @@ def add_scaled_rmsnorm(resid, terms, gain, eps, out, rows=None):
 
 def _grouped(name, a, lda, a_group, w, w_group, ldw, out, ldo, o_group, M, N, K, groups, seg=None, a_rows=None,
              o_rows=None, row_weight=None, gate=None, gate_ld=0, gate_group=0, gate_col=0, act=0, rows_bound=0,
-             force_simt=False, w_packed=False):
+             force_simt=False, w_packed=False, pair=None):
     L = ctypes.c_long
     _call(load_library("core"), "syn_grouped_product", _ptr(a), L(lda), L(a_group), _ptr(w), L(w_group), L(ldw), _ptr(out),
           L(ldo), L(o_group), _is_f32(a), _is_f32(out), _ptr(seg), _ptr(a_rows), _ptr(o_rows), _ptr(row_weight), _ptr(gate),
           L(gate_ld), L(gate_group), int(gate_col), int(act), int(M), int(N), int(K), int(groups), int(rows_bound),
-          int(force_simt), int(bool(w_packed)), _stream())
+          int(force_simt), int(bool(w_packed)), *((0, ctypes.c_float(0.0)) if pair is None else (pair[0] + 1, pair[1])),
+          _stream())
 
 
 def heads_product(x, w, out, out_offset=0, gate=None, gate_per_value=True, force_simt=False):
@@ -1354,12 +1356,21 @@ def pack_expert_weights(w):
     return w.view(E, J // 16, 16, K // 32, 4, 8).permute(0, 1, 3, 4, 2, 5).reshape(E, J // 16, K // 32, 64, 8).contiguous()
 
 
-def experts_product(x, w, out, seg, a_rows, o_rows, row_weight=None, gelu=False, force_simt=False):
+def pair_expert_rows(gate, up):
+    """Gate and up matrices [E, J, K] as one [E, 2 J, K] whose rows alternate (2 j: gate row j, 2 j + 1: up row j): what
+    experts_product(gated=...) multiplies with."""
+    E, J, K = gate.shape
+    return torch.stack([gate, up], 2).reshape(E, 2 * J, K).contiguous()
+
+
+def experts_product(x, w, out, seg, a_rows, o_rows, row_weight=None, gelu=False, force_simt=False, gated=None):
     """out[o_rows[r]] = epilogue(x[a_rows[r]] . w[e]^T) for the places r of each expert e's segment.  x [*, K] in the
     engine's type, w [E, J, K] in that type (or bf16 in fragment order, pack_expert_weights: five dimensions), out
     [*, J] in that type or float; the index lists come from route_sort and
     must stay inside x and out (the caller sees to that: they are on the device).  Epilogue: the exact GELU, then the
-    row's weight, each if asked for.  force_simt: as in heads_product."""
+    row's weight, each if asked for.  gated: an activation of the gated products (ACTIVATIONS; one with a bound as the
+    pair (name, bound)): w then holds gate and up rows in turns (pair_expert_rows), and out [*, J / 2] receives the
+    activation of each pair of sums.  force_simt: as in heads_product."""
     _need(x, "experts_product.x", (_BF16, _F32), (None, None))
     K = x.shape[1]
     packed = isinstance(w, torch.Tensor) and w.dim() == 5
@@ -1370,15 +1381,21 @@ def experts_product(x, w, out, seg, a_rows, o_rows, row_weight=None, gelu=False,
     else:
         _need(w, "experts_product.w", x.dtype, (None, None, K))
         E, J = w.shape[0], w.shape[1]
-    _need(out, "experts_product.out", (x.dtype, _F32), (None, J))
+    pair = None
+    if gated is not None:
+        if gelu or J % 2:
+            raise KernelError(f"experts_product: a gated activation over {J} rows in pairs, and no other activation")
+        pair = _activation_args(gated)
+    _need(out, "experts_product.out", (x.dtype, _F32), (None, J // 2 if pair else J))
     _need(seg, "experts_product.seg", _I32, (E + 1,))
     _need(a_rows, "experts_product.a_rows", _I32, (None,))
     P = a_rows.shape[0]
     _need(o_rows, "experts_product.o_rows", _I32, (P,))
     if row_weight is not None:
         _need(row_weight, "experts_product.row_weight", _F32, (P,))
-    _grouped("experts_product", x, K, 0, w, J * K, K, out, J, 0, P, J, K, E, seg=seg, a_rows=a_rows, o_rows=o_rows,
-             row_weight=row_weight, act=1 if gelu else 0, rows_bound=P, force_simt=force_simt, w_packed=packed)
+    _grouped("experts_product", x, K, 0, w, J * K, K, out, J // 2 if pair else J, 0, P, J, K, E, seg=seg, a_rows=a_rows,
+             o_rows=o_rows, row_weight=row_weight, act=1 if gelu else 0, rows_bound=P, force_simt=force_simt,
+             w_packed=packed, pair=pair)
 
 
 # ----------------------------------------------------------------------------- latent attention: intake

@@ -152,9 +152,9 @@ class RoutedExperts(FeedForward):
         p, (up, down, router, bias) = self.prefix, self.names[:4]
         # every expert's matrices kept once: in fragment order where type and sizes allow, else in plain rows
         if self.n_experts:
-            if self.gated:      # an expert's gate rows, then its up rows: one product for both
-                w_up = torch.stack([torch.cat([get(p + self.names[4].format(e)), get(p + up.format(e))], 0)
-                                    for e in range(self.n_experts)]).contiguous()
+            if self.gated:      # an expert's gate and up rows in turns: one product for both, the activation its epilogue
+                w_up = ops.pair_expert_rows(torch.stack([get(p + self.names[4].format(e)) for e in range(self.n_experts)]),
+                                            torch.stack([get(p + up.format(e)) for e in range(self.n_experts)]))
             else:
                 w_up = torch.stack([get(p + up.format(e)) for e in range(self.n_experts)]).contiguous()
             packed = ops.pack_expert_weights(w_up)
@@ -191,9 +191,7 @@ class RoutedExperts(FeedForward):
             real = seg[:self.n_experts + 1]          # the experts with matrices come first
             mid = torch.empty((N * self.top, self.ff), dtype=h.dtype, device=dev)
             if self.gated:
-                both = torch.empty((N * self.top, 2 * self.ff), dtype=h.dtype, device=dev)
-                ops.experts_product(h, self.w_up, both, real, tok_of, pair_of)
-                ops.swiglu(both, mid, self.activation)
+                ops.experts_product(h, self.w_up, mid, real, tok_of, pair_of, gated=self.activation)
             else:
                 ops.experts_product(h, self.w_up, mid, real, tok_of, pair_of, gelu=True)
             ops.experts_product(mid, self.w_down, y.view(self.top * N, self.hidden), real, pair_of, part_of,

@@ -30,7 +30,7 @@ def attn(heads, kv_heads, dim, vdim, conv, window=None, dims=None, base=10000.0,
     return "attention", m
 
 
-def moe(ff, experts, top, identity=0, groups=None, limit=1.5, shared=None):
+def moe(ff, experts, top, identity=0, groups=None, limit=1.25, shared=None):
     router = {"experts": experts, "top": top}
     if identity:
         router["identity"] = identity
@@ -60,7 +60,7 @@ def config(vocab, width, layers, eps=1e-6, scale=None, rank=8):
 # S: one head everywhere, windows of one and of two, one expert beside one identity, the top one of them only: a choice
 #    that the rounding of bfloat16 activations can turn changes a token's result altogether, so this one is 32-bit only.
 CONFIGS = {
-    "P": config(300, 64, [(attn(4, 2, 16, 24, 3, window=20, dims=8, scaling=(4.0, 64, 16.0, 2.0)), moe(32, 6, 3, identity=2, groups=(4, 2), shared=(48, 1.0))),
+    "P": config(300, 64, [(attn(4, 2, 16, 24, 3, window=20, dims=8, scaling=(4.0, 64, 16.0, 2.0)), moe(32, 6, 3, identity=2, groups=(4, 2), shared=(48, 0.9))),
                           (ssm(4, 16, 24, 2, 4, norm_groups=2), None),
                           (delta(4, 2, 16, 24, 3), moe(24, 4, 2, identity=1, limit=0.7, shared=(16, 2.0))),
                           (ssm(6, 8, 20, 3, 2, norm_groups=3), moe(32, 6, 3, identity=2, groups=(2, 1)))], scale=4.0),
@@ -69,7 +69,7 @@ CONFIGS = {
                           (delta(3, 1, 12, 20, 5), None),
                           (attn(2, 1, 20, 6, 1, window=65, dims=4, base=500.0, diff=0.8), moe(12, 2, 1, identity=2, groups=(2, 2)))],
                 eps=1e-5, rank=5),
-    "R": config(512, 128, [(delta(4, 4, 64, 64, 4), moe(64, 16, 4, groups=(4, 2), shared=(96, 1.0))),
+    "R": config(512, 128, [(delta(8, 4, 64, 32, 3), moe(64, 16, 4, groups=(4, 2), shared=(80, 1.1))),
                            (attn(4, 2, 32, 64, 3, window=4096, dims=32, scaling=(8.0, 128, 32.0, 1.0)), moe(64, 8, 2, identity=0)),
                            (ssm(8, 32, 128, 2, 4, norm_groups=4), moe(32, 6, 2, identity=2, shared=(64, 1.5))),
                            (attn(8, 2, 64, 32, 2, dims=16, base=1e6), None)], scale=11.3, rank=16),

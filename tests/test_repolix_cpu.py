@@ -158,9 +158,9 @@ def test_plain_router():
 def test_plain_experts_and_the_whole_model_runs():
     h = torch.tensor([[10.0, -10.0]], dtype=F64)
     eye = torch.eye(2, dtype=F64)
-    y = P.clamped_expert(h, eye, eye, eye, 1.5)
-    g = torch.tensor([1.5, -10.0], dtype=F64)
-    u = torch.tensor([1.5, -1.5], dtype=F64)
+    y = P.clamped_expert(h, eye, eye, eye, 1.25)
+    g = torch.tensor([1.25, -10.0], dtype=F64)
+    u = torch.tensor([1.25, -1.25], dtype=F64)
     assert torch.allclose(y[0], g * torch.sigmoid(1.702 * g) * (u + 1.0))
     toks = tokens_for("P", 30, 1)
     res, lg = plain_model("P").residuals(toks)

@@ -238,6 +238,7 @@ __global__ void __launch_bounds__(256) grouped_product_mfma_kernel(GroupedArgs g
 #define GT_BN 128
 #define GT_BK 64
 #define GT_LD (GT_BK + 8)
+template <bool PAIR>
 __global__ void __launch_bounds__(256) grouped_product_tiled_kernel(GroupedArgs g) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];      // [2][(GT_BM + GT_BN) * GT_LD]
   const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
@@ -347,7 +348,7 @@ __global__ void __launch_bounds__(256) grouped_product_tiled_kernel(GroupedArgs 
       for (int e = 0; e < 16; ++e) {
         const int r = row0 + wm + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
         const int n = n0 + wn + j * 32 + lane % 32;
-        if (g.pair) {      // (neighbouring lanes hold neighbouring outputs: the even lane takes its neighbour's up sum)
+        if constexpr (PAIR) {      // (neighbouring lanes hold neighbouring outputs: the even lane takes its neighbour's up sum)
           const float up = __shfl_xor(acc[i][j][e], 1, SYN_WAVE);
           if (lane % 2 == 0 && r < row_end && n < g.N) grouped_store(g, r, b, n / 2, grouped_pair(g, acc[i][j][e], up, r));
         } else if (r < row_end && n < g.N) {
@@ -388,10 +389,14 @@ SYN_EXPORT int syn_grouped_product(const void* a, long lda, long a_group, const 
     const size_t lds = (size_t)2 * (GT_BM + GT_BN) * GT_LD * sizeof(bf16);
     static OncePerDevice raised;
     const hipError_t e = once_per_device(raised, [&] {
-      return hipFuncSetAttribute((const void*)grouped_product_tiled_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      const hipError_t r = hipFuncSetAttribute((const void*)grouped_product_tiled_kernel<false>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      return r != hipSuccess ? r : hipFuncSetAttribute((const void*)grouped_product_tiled_kernel<true>,
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     });
     SYN_CHECK(e == hipSuccess, "grouped_product: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
-    grouped_product_tiled_kernel<<<grid, 256, lds, stream>>>(g);
+    if (pair) grouped_product_tiled_kernel<true><<<grid, 256, lds, stream>>>(g);
+    else grouped_product_tiled_kernel<false><<<grid, 256, lds, stream>>>(g);
   } else if (!in_is_f32 && aligned && force_simt != 1) {
     const int row_tiles = seg_start ? (rows_bound + GP_TM - 1) / GP_TM + groups : (M + GP_TM - 1) / GP_TM;
     const long wide = (long)row_tiles * ((N + 255) / 256) * (seg_start ? 1 : groups);

@@ -1,14 +1,17 @@
 // Attention over the paged cache for mixers whose scores, mask and softmax differ from the plain causal ones:
 //
 //   score(i, j) = scale (q_i . k_j) [soft cap] - slope_h (i - j) - r1_h ln(1 + r2_h (i - j))
-//   key j is visible to the query at i iff  j <= i  and  (window <= 0 or i - j < window or j < keep_first):
-//       a sliding window that never loses the first keep_first keys, which keep their true positions;
-//   p_j = exp(score_j) / (sink + sum_j exp(score_j)),  sink = 1 with `sink_one` (a further key of score 0 that has
-//       no value), else 0;
+//   key j is visible to the query at i iff  j <= i  and  (window <= 0 or i - j < window or j < keep_first)
+//       and (chunk <= 0 or j / chunk == i / chunk or j < keep_first):
+//       a sliding window that never loses the first keep_first keys, which keep their true positions, and/or runs of
+//       `chunk` positions counted from the sequence's first token, whose keys only their own run's queries see;
+//   p_j = exp(score_j) / (sink + sum_j exp(score_j)),  sink = exp(sinks[h]) with `sinks` (a learned score a head of a
+//       further key that has no value), 1 with `sink_one` (that score is 0), else 0;
 //   head h reads kv head h / (heads / kv heads); keys have `dim` values, values `vdim`;
 //   v_share > 1: that many neighbouring kv heads read the values of one value head (kv heads / v_share of them are
 //       stored), as the maps of a differential attention do, which have keys of their own and the values in common;
-//   the heads' results may be multiplied by sigmoid(gate) before they are stored.
+//   the heads' results may be multiplied by sigmoid(gate) before they are stored: a gate for every value, or with
+//       `gate_per_head` one for each head.
 // Scores, weights and sums are 32-bit whatever the cache's type; the weights are not rounded before they meet V.
 //
 // Cache pages hold 64 tokens: k_pages[page, kv_head, token, dim], v_pages[page, kv_head, vdim, token] (plain rows in
@@ -27,21 +30,32 @@ struct WindowTerms {
   int keep_first;
   int sink_one;
   int v_share;           // this many neighbouring kv heads read one value head (1: each its own)
+  const float* sinks;    // [heads] or nullptr: the score of a key without a value in every softmax
+  int chunk;             // 0: none
+  int gate_per_head;     // the gate's rows hold one number a head (else one for each value)
 };
+
+// the first key that the query at `pos` sees (kept first keys aside); it never falls as pos grows
+__device__ __forceinline__ int first_visible(int pos, const WindowTerms& t) {
+  int lo = t.window > 0 ? max(0, pos - t.window + 1) : 0;
+  if (t.chunk > 0) lo = max(lo, pos / t.chunk * t.chunk);
+  return lo;
+}
 
 // ---------------------------------------------------------------- intake: bias, q/k norm, cache write
 // proj [N][width] float holds the fused projection  [q heads x dim | k heads x dim | v heads x vdim | ...]; what lies
 // behind v (a gate) is left where it is.  One wave for each (token, q head | k head | v head); there are nv value
 // heads (nkv, unless several kv heads share a value head).
 // cos_t, sin_t [positions][rot / 2] (or null): after the norm the first `rot` values of a q or k head are turned, value
-// i < rot / 2 paired with value i + rot / 2, by the angle whose cosine and sine stand at [position][i].
+// i < rot / 2 paired with value i + rot / 2 (with `pairs`: value 2 i with value 2 i + 1), by the angle whose cosine
+// and sine stand at [position][i].  Without write_kv the rows hold queries only (keys and values are another layer's).
 template <typename T>
 __global__ void window_intake_kernel(const float* __restrict__ proj, int width, const float* __restrict__ bias,
                                      T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
                                      const int* __restrict__ page_table, int table_stride,
                                      const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                      const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
-                                     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
+                                     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, int pairs,
                                      int nh, int nkv, int nv, int dim, int vdim, int write_kv) {
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
   const int tok = blockIdx.x;
@@ -81,11 +95,13 @@ __global__ void window_intake_kernel(const float* __restrict__ proj, int width, 
     float v = src[d] + (b ? b[d] : 0.f);
     if (gain) v = v * inv * gain[d];
     if (d < 2 * half) {
-      const int i = d < half ? d : d - half, mate = d < half ? d + half : d - half;
+      const bool first = pairs ? d % 2 == 0 : d < half;
+      const int i = pairs ? d / 2 : (first ? d : d - half);
+      const int mate = pairs ? (d ^ 1) : (first ? d + half : d - half);
       float o = src[mate] + (b ? b[mate] : 0.f);
       if (gain) o = o * inv * gain[mate];
       const float c = cos_t[(size_t)pos * half + i], sn = sin_t[(size_t)pos * half + i];
-      v = d < half ? v * c - o * sn : v * c + o * sn;
+      v = first ? v * c - o * sn : v * c + o * sn;
     }
     dst[(size_t)d * stride] = from_f32<T>(v);
   }
@@ -94,10 +110,11 @@ __global__ void window_intake_kernel(const float* __restrict__ proj, int width, 
 SYN_EXPORT int syn_window_intake(const float* proj, int width, const float* bias, void* q_out, void* k_pages,
                                  void* v_pages, int is_f32, const int* page_table, int table_stride, const int* tok_seq,
                                  const int* tok_pos, const float* q_gain, const float* k_gain, float eps,
-                                 const float* cos_t, const float* sin_t, int rot, int n_tokens,
+                                 const float* cos_t, const float* sin_t, int rot, int pairs, int n_tokens,
                                  int nh, int nkv, int nv, int dim, int vdim, int write_kv, hipStream_t stream) {
   SYN_CHECK(n_tokens > 0 && nh > 0 && nkv > 0 && nv > 0 && dim > 0 && vdim > 0, "window_intake: empty input");
-  SYN_CHECK(width >= (nh + nkv) * dim + nv * vdim, "window_intake: rows of %d values do not hold q, k and v", width);
+  SYN_CHECK(width >= (write_kv ? (nh + nkv) * dim + nv * vdim : nh * dim), "window_intake: rows of %d values do not hold q%s",
+            width, write_kv ? ", k and v" : "");
   SYN_CHECK((q_gain == nullptr) == (k_gain == nullptr), "window_intake: q and k gains come together");
   SYN_CHECK((cos_t == nullptr) == (sin_t == nullptr) && (cos_t == nullptr || (rot > 0 && rot % 2 == 0 && rot <= dim)),
             "window_intake: a rotation of %d of %d values", rot, dim);
@@ -106,13 +123,13 @@ SYN_EXPORT int syn_window_intake(const float* proj, int width, const float* bias
   if (is_f32)
     window_intake_kernel<float><<<grid, wpb * SYN_WAVE, 0, stream>>>(proj, width, bias, (float*)q_out, (float*)k_pages,
                                                                      (float*)v_pages, page_table, table_stride, tok_seq,
-                                                                     tok_pos, q_gain, k_gain, eps, cos_t, sin_t, rot, nh,
-                                                                     nkv, nv, dim, vdim, write_kv);
+                                                                     tok_pos, q_gain, k_gain, eps, cos_t, sin_t, rot, pairs,
+                                                                     nh, nkv, nv, dim, vdim, write_kv);
   else
     window_intake_kernel<bf16><<<grid, wpb * SYN_WAVE, 0, stream>>>(proj, width, bias, (bf16*)q_out, (bf16*)k_pages,
                                                                     (bf16*)v_pages, page_table, table_stride, tok_seq,
-                                                                    tok_pos, q_gain, k_gain, eps, cos_t, sin_t, rot, nh,
-                                                                    nkv, nv, dim, vdim, write_kv);
+                                                                    tok_pos, q_gain, k_gain, eps, cos_t, sin_t, rot, pairs,
+                                                                    nh, nkv, nv, dim, vdim, write_kv);
   SYN_LAUNCH_CHECK("window_intake");
   return 0;
 }
@@ -163,16 +180,17 @@ window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, 
   for (int d = threadIdx.x; d < dim; d += WAVES * SYN_WAVE) qs[d] = to_f32<T>(qr[d]);
   __syncthreads();
 
-  const int lo = terms.window > 0 ? max(0, pos - terms.window + 1) : 0;
+  const int lo = first_visible(pos, terms);
   const int kept = min(terms.keep_first, lo);        // keys below `kept` are seen although the window has passed them
   const int n_kept_blocks = kept > 0 ? (kept - 1) / SYN_PAGE + 1 : 0;
   const int first_window_block = max(lo / SYN_PAGE, n_kept_blocks);
   const int n_blocks = n_kept_blocks + (pos / SYN_PAGE - first_window_block + 1);
   const float slope = terms.slopes ? terms.slopes[head] : 0.f;
   const float r1 = terms.r1 ? terms.r1[head] : 0.f, r2 = terms.r1 ? terms.r2[head] : 0.f;
-  // the sink is a key of score 0 without a value: the first wave's running maximum and sum start from it
-  const bool sink_here = terms.sink_one && wave == 0;
-  float m = sink_here ? 0.f : -INFINITY, l = sink_here ? 1.f : 0.f;
+  // the sink is a key without a value whose score is sinks[head], or 0: the first wave's running maximum and sum
+  // start from it
+  const bool sink_here = (terms.sink_one || terms.sinks) && wave == 0;
+  float m = sink_here ? (terms.sinks ? terms.sinks[head] : 0.f) : -INFINITY, l = sink_here ? 1.f : 0.f;
   float o[MAXD / SYN_WAVE] = {};
   for (int idx = wave; idx < n_blocks; idx += WAVES) {
     const int kb = idx < n_kept_blocks ? idx : first_window_block + (idx - n_kept_blocks);
@@ -251,14 +269,15 @@ window_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, 
     }
   }
   T* orow = out + ((size_t)tok * nh + head) * vdim;
-  const float* g = gate ? gate + (size_t)tok * gate_stride + (size_t)head * vdim : nullptr;
+  const int per_head = terms.gate_per_head;
+  const float* g = gate ? gate + (size_t)tok * gate_stride + (per_head ? head : (size_t)head * vdim) : nullptr;
 #pragma unroll
   for (int i = 0; i < MAXD / SYN_WAVE; ++i) {
     const int d = lane + i * SYN_WAVE;
     if (d < vdim) {
       float v = o[i] / l;
       if (g) {
-        const float z = g[d] + (gate_bias ? gate_bias[head * vdim + d] : 0.f);
+        const float z = g[per_head ? 0 : d] + (gate_bias ? gate_bias[per_head ? head : head * vdim + d] : 0.f);
         v *= 1.f / (1.f + expf(-z));
       }
       orow[d] = from_f32<T>(v);
@@ -272,8 +291,10 @@ SYN_EXPORT int syn_window_attention(const void* q, const void* k_pages, const vo
                                     const float* gate, int gate_stride, const float* gate_bias, void* out, float scale,
                                     int n_tokens, int nh, int nkv, int dim, int vdim, const float* slopes,
                                     const float* r1, const float* r2, float softcap, int window, int keep_first,
-                                    int sink_one, int v_share, hipStream_t stream) {
+                                    int sink_one, int v_share, const float* sinks, int chunk, int gate_per_head,
+                                    hipStream_t stream) {
   SYN_CHECK(n_tokens > 0 && nh > 0 && nkv > 0, "window_attention: empty input");
+  SYN_CHECK(chunk >= 0 && !(sinks && sink_one), "window_attention: chunks of %d, or two sinks", chunk);
   SYN_CHECK(v_share > 0 && nkv % v_share == 0, "window_attention: %d kv heads in shares of %d", nkv, v_share);
   SYN_CHECK(nh % nkv == 0, "window_attention: %d heads do not divide into %d kv heads", nh, nkv);
   SYN_CHECK(dim > 0 && dim <= AW_MAX_DIM && vdim > 0 && vdim <= AW_MAX_DIM,
@@ -281,8 +302,9 @@ SYN_EXPORT int syn_window_attention(const void* q, const void* k_pages, const vo
   SYN_CHECK(softcap >= 0.f && window >= 0 && keep_first >= 0, "window_attention: soft cap %g, window %d, kept %d",
             (double)softcap, window, keep_first);
   SYN_CHECK((r1 == nullptr) == (r2 == nullptr), "window_attention: r1 and r2 come together");
-  SYN_CHECK(gate == nullptr || gate_stride >= nh * vdim, "window_attention: gate rows of %d values", gate_stride);
-  const WindowTerms terms = {slopes, r1, r2, softcap, window, keep_first, sink_one, v_share};
+  SYN_CHECK(gate == nullptr || gate_stride >= (gate_per_head ? nh : nh * vdim), "window_attention: gate rows of %d values",
+            gate_stride);
+  const WindowTerms terms = {slopes, r1, r2, softcap, window, keep_first, sink_one, v_share, sinks, chunk, gate_per_head};
   const dim3 grid(n_tokens, nh);
   // few (token, head) pairs (single tokens of a few sequences): eight waves share each pair's keys
   const bool many_waves = (long)n_tokens * nh < 8L * syn_compute_units();
@@ -371,12 +393,12 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
     for (int s = 0; s < AWP_TILES; ++s)
       if (s < dim / 16) qf4[s] = *(const bf16x4*)(qrow + 16 * s + 4 * g);
   }
-  const int W = terms.window;
-  const int lo_q = W > 0 ? max(0, qpos - W + 1) : 0;                          // this lane's query
-  const int lo_wave = W > 0 ? max(0, past + n0 - W + 1) : 0;                  // this wave's first query
+  const int lo_q = first_visible(qpos, terms);                                // this lane's query
+  const int lo_wave = first_visible(past + n0, terms);                        // this wave's first query
   const int kmax_wave = past + min(n0 + 15, n_new - 1);
+  const int lo_last = first_visible(kmax_wave, terms);                        // this wave's last query
   // the pages that the workgroup's 64 queries see together
-  const int lo_first = W > 0 ? max(0, past + nb - W + 1) : 0;
+  const int lo_first = first_visible(past + nb, terms);
   const int kmax = past + min(nb + 63, n_new - 1);
   const int kept = min(terms.keep_first, lo_first);
   const int n_kept_blocks = kept > 0 ? (kept - 1) / SYN_PAGE + 1 : 0;
@@ -386,7 +408,9 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
   const float r1 = terms.r1 ? terms.r1[head] : 0.f, r2 = terms.r1 ? terms.r2[head] : 0.f;
   constexpr float LOG2E = 1.4426950408889634f;
   const float scale2 = scale * LOG2E, slope2 = slope * LOG2E, cap2 = terms.softcap * LOG2E;
-  float m = terms.sink_one ? 0.f : -INFINITY, l = terms.sink_one ? 1.f : 0.f;     // (the sink's score 0 is 0 in any unit)
+  // (the sink's score in units of ln 2; a score of 0 is 0 in any unit)
+  float m = terms.sinks ? terms.sinks[head] * LOG2E : (terms.sink_one ? 0.f : -INFINITY);
+  float l = (terms.sinks || terms.sink_one) ? 1.f : 0.f;
   f32x4 O[AWP_TILES];
 #pragma unroll
   for (int j = 0; j < AWP_TILES; ++j) O[j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -450,8 +474,8 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
       }
     }
     // the terms and the mask on this lane's 16 scores (keys 16 t + 4 g + e of the page, all of query i); a page that
-    // lies behind the wave's first query and inside its last query's window is seen whole by all of them: no mask
-    const bool whole = page_hi <= past + n0 && (W <= 0 || page_lo >= kmax_wave - W + 1);
+    // lies behind the wave's first query and inside its last query's window and chunk is seen whole by all of them: no mask
+    const bool whole = page_hi <= past + n0 && page_lo >= lo_last;
     const float dist0 = (float)(qpos - page_lo - 4 * g);
     // scores in units of ln 2 from here on (scale, slope and cap carry log2 e; r1 ln(x) = r1 log2(x) ln 2): the
     // exponentials below are bare exp2
@@ -527,7 +551,8 @@ window_prefill_bf16_kernel(const bf16* __restrict__ q, const bf16* __restrict__ 
       for (int e = 0; e < 4; ++e) {
         float v = O[j][e] * inv;
         if (gate) {
-          const float z = gate[tok * gate_stride + col + e] + (gate_bias ? gate_bias[col + e] : 0.f);
+          const int at = terms.gate_per_head ? head : col + e;
+          const float z = gate[tok * gate_stride + at] + (gate_bias ? gate_bias[at] : 0.f);
           v *= 1.f / (1.f + __expf(-z));
         }
         o4[e] = (bf16)v;
@@ -545,7 +570,8 @@ SYN_EXPORT int syn_window_attention_prefill_bf16(const void* q, const void* k_pa
                                                  int gate_stride, const float* gate_bias, void* out, float scale, int nh,
                                                  int nkv, int dim, int vdim, const float* slopes, const float* r1,
                                                  const float* r2, float softcap, int window, int keep_first, int sink_one,
-                                                 int v_share, hipStream_t stream) {
+                                                 int v_share, const float* sinks, int chunk, int gate_per_head,
+                                                 hipStream_t stream) {
   SYN_CHECK(n_tokens > 0 && n_seqs > 0 && nh > 0 && nkv > 0, "window_attention_prefill: empty input");
   SYN_CHECK(v_share > 0 && nkv % v_share == 0, "window_attention_prefill: %d kv heads in shares of %d", nkv, v_share);
   SYN_CHECK(nh % nkv == 0, "window_attention_prefill: %d heads do not divide into %d kv heads", nh, nkv);
@@ -554,11 +580,12 @@ SYN_EXPORT int syn_window_attention_prefill_bf16(const void* q, const void* k_pa
   SYN_CHECK(softcap >= 0.f && window >= 0 && keep_first >= 0, "window_attention_prefill: soft cap %g, window %d, kept %d",
             (double)softcap, window, keep_first);
   SYN_CHECK((r1 == nullptr) == (r2 == nullptr), "window_attention_prefill: r1 and r2 come together");
-  SYN_CHECK(gate == nullptr || (gate_stride >= nh * vdim && gate_stride % 4 == 0 && (uintptr_t)gate % 16 == 0),
-            "window_attention_prefill: gate rows of %d values", gate_stride);
+  SYN_CHECK(gate == nullptr || gate_stride >= (gate_per_head ? nh : nh * vdim), "window_attention_prefill: gate rows of %d values",
+            gate_stride);
+  SYN_CHECK(chunk >= 0 && !(sinks && sink_one), "window_attention_prefill: chunks of %d, or two sinks", chunk);
   SYN_CHECK((uintptr_t)q % 16 == 0 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0 && (uintptr_t)out % 8 == 0,
             "window_attention_prefill: operands are not aligned");
-  const WindowTerms terms = {slopes, r1, r2, softcap, window, keep_first, sink_one, v_share};
+  const WindowTerms terms = {slopes, r1, r2, softcap, window, keep_first, sink_one, v_share, sinks, chunk, gate_per_head};
   const dim3 grid((n_tokens + 63) / 64 + n_seqs, nh);      // at most this many tiles of 64 queries; the rest leave at once
   if (dim % 32 == 0)
     window_prefill_bf16_kernel<true><<<grid, 256, 0, stream>>>(

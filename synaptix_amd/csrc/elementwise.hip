@@ -646,16 +646,21 @@ SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_o
 // ------------------------------------------------------------------ residual sum of scaled terms + RMSNorm
 // A layer whose sublayers run side by side on one normed input leaves up to two results, each with a scale of its
 // own for every channel:   x[r] += s1 * d1[r] + s2 * d2[r]   (s: float [H], d: n_parts partial sums [parts][rows][H]
-// added in order, or null), then out[r] = norm(x[r]) * gain if `out` is given.  With `rows` only those rows are summed
+// added in order, or null), then out[r] = norm(x[r]) * gain if `out` is given.  A term may also carry a gate for every
+// row (g: one float a row at g[r * stride], or null): the term is then multiplied by sigmoid(g[r]).  With `rows` only those rows are summed
 // and normed, and x stays as it is.  32-bit throughout; one rounding at the store.
 template <typename TOut>
 __global__ void add_scaled_rmsnorm_kernel(float* __restrict__ resid, const int* __restrict__ rows, size_t part_stride,
                                           const float* __restrict__ d1, int parts1, const float* __restrict__ s1,
                                           const float* __restrict__ d2, int parts2, const float* __restrict__ s2,
-                                          const void* __restrict__ gain, int gain_is_f32, float eps,
+                                          const float* __restrict__ g1, int g1_stride, const float* __restrict__ g2,
+                                          int g2_stride, const void* __restrict__ gain, int gain_is_f32, float eps,
                                           TOut* __restrict__ out, int H) {
   __shared__ float red[16];
   const int r = rows ? rows[blockIdx.x] : blockIdx.x;
+  // a term's factor for the whole row: the sigmoid of one number a row (or 1)
+  const float f1 = g1 ? 1.f / (1.f + expf(-g1[(size_t)r * g1_stride])) : 1.f;
+  const float f2 = g2 ? 1.f / (1.f + expf(-g2[(size_t)r * g2_stride])) : 1.f;
   float* x = resid + (size_t)r * H;
   const float* a = d1 ? d1 + (size_t)r * H : nullptr;
   const float* b = d2 ? d2 + (size_t)r * H : nullptr;
@@ -665,12 +670,12 @@ __global__ void add_scaled_rmsnorm_kernel(float* __restrict__ resid, const int* 
     if (a) {
       float t = 0.f;
       for (int p = 0; p < parts1; ++p) t += a[p * part_stride + i];
-      v = fmaf(s1 ? s1[i] : 1.f, t, v);
+      v = fmaf(s1 ? s1[i] * f1 : f1, t, v);
     }
     if (b) {
       float t = 0.f;
       for (int p = 0; p < parts2; ++p) t += b[p * part_stride + i];
-      v = fmaf(s2 ? s2[i] : 1.f, t, v);
+      v = fmaf(s2 ? s2[i] * f2 : f2, t, v);
     }
     return v;
   };
@@ -691,7 +696,8 @@ __global__ void add_scaled_rmsnorm_kernel(float* __restrict__ resid, const int* 
 }
 
 SYN_EXPORT int syn_add_scaled_rmsnorm(float* resid, int n_rows, const int* rows, int n_out, const float* d1, int parts1,
-                                      const float* s1, const float* d2, int parts2, const float* s2, const void* gain,
+                                      const float* s1, const float* d2, int parts2, const float* s2, const float* g1,
+                                      int g1_stride, const float* g2, int g2_stride, const void* gain,
                                       int gain_is_f32, float eps, void* out, int out_is_f32, int H, hipStream_t stream) {
   SYN_CHECK(n_out > 0 && H > 0 && n_rows > 0, "add_scaled_rmsnorm: empty input (%d rows, width %d)", n_out, H);
   SYN_CHECK(parts1 >= 1 && parts1 <= 64 && parts2 >= 1 && parts2 <= 64, "add_scaled_rmsnorm: %d and %d partial sums", parts1, parts2);
@@ -699,10 +705,12 @@ SYN_EXPORT int syn_add_scaled_rmsnorm(float* resid, int n_rows, const int* rows,
   const size_t stride = (size_t)n_rows * H;
   const int block = H >= 4096 ? 1024 : (H >= 1024 ? 512 : 256);
   if (out_is_f32)
-    add_scaled_rmsnorm_kernel<float><<<n_out, block, 0, stream>>>(resid, rows, stride, d1, parts1, s1, d2, parts2, s2, gain,
+    add_scaled_rmsnorm_kernel<float><<<n_out, block, 0, stream>>>(resid, rows, stride, d1, parts1, s1, d2, parts2, s2, g1,
+                                                                  g1_stride, g2, g2_stride, gain,
                                                                   gain_is_f32, eps, (float*)out, H);
   else
-    add_scaled_rmsnorm_kernel<bf16><<<n_out, block, 0, stream>>>(resid, rows, stride, d1, parts1, s1, d2, parts2, s2, gain,
+    add_scaled_rmsnorm_kernel<bf16><<<n_out, block, 0, stream>>>(resid, rows, stride, d1, parts1, s1, d2, parts2, s2, g1,
+                                                                  g1_stride, g2, g2_stride, gain,
                                                                  gain_is_f32, eps, (bf16*)out, H);
   SYN_LAUNCH_CHECK("add_scaled_rmsnorm");
   return 0;

@@ -484,7 +484,8 @@ SYN_EXPORT int syn_route_topk(const float* logits, const float* bias, int* ids, 
 // divided by their sum.  One wave a token.
 __global__ void __launch_bounds__(256) route_scores_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
                                                            int* __restrict__ ids, float* __restrict__ weights, int n_tokens,
-                                                           int E, int top, int n_groups, int keep_groups, int renorm) {
+                                                           int E, int ld, int top, int n_groups, int keep_groups, int renorm,
+                                                           float scale) {
   __shared__ float ss[4][ROUTE_MAX_EXPERTS];       // the scores
   __shared__ float cs[4][ROUTE_MAX_EXPERTS];       // the choice scores
   __shared__ float gs[4][ROUTE_MAX_EXPERTS];       // the groups' scores
@@ -501,11 +502,11 @@ __global__ void __launch_bounds__(256) route_scores_kernel(const float* __restri
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   };
   float mx = -INFINITY;
-  for (int e = lane; e < E; e += SYN_WAVE) mx = fmaxf(mx, logits[(size_t)tok * E + e]);
+  for (int e = lane; e < E; e += SYN_WAVE) mx = fmaxf(mx, logits[(size_t)tok * ld + e]);
   mx = wave_max(mx);
   float sum = 0.f;
   for (int e = lane; e < E; e += SYN_WAVE) {
-    const float p = expf(logits[(size_t)tok * E + e] - mx);
+    const float p = expf(logits[(size_t)tok * ld + e] - mx);
     sc[e] = p;
     sum += p;
   }
@@ -559,20 +560,23 @@ __global__ void __launch_bounds__(256) route_scores_kernel(const float* __restri
       total = 0.f;
       for (int t = 0; t < top; ++t) total += chosen[t];
     }
-    for (int t = 0; t < top; ++t) weights[(size_t)tok * top + t] = chosen[t] / total;
+    for (int t = 0; t < top; ++t) weights[(size_t)tok * top + t] = chosen[t] / total * scale;
   }
 }
 
+// logits: rows of `ld` values whose first E are the router's outputs; weights: the chosen scores (over their sum with
+// renorm) times `scale`
 SYN_EXPORT int syn_route_scores(const float* logits, const float* correction, int* ids, float* weights, int n_tokens, int E,
-                                int top, int n_groups, int keep_groups, int renorm, hipStream_t stream) {
+                                int ld, int top, int n_groups, int keep_groups, int renorm, float scale, hipStream_t stream) {
+  SYN_CHECK(ld >= E, "route_scores: rows of %d values for %d experts", ld, E);
   SYN_CHECK(n_tokens > 0, "route_scores: empty input");
   SYN_CHECK(E > 0 && E <= ROUTE_MAX_EXPERTS, "route_scores: %d experts (at most %d)", E, ROUTE_MAX_EXPERTS);
   SYN_CHECK(n_groups > 0 && E % n_groups == 0 && keep_groups > 0 && keep_groups <= n_groups,
             "route_scores: %d experts in %d groups of which %d stay", E, n_groups, keep_groups);
   SYN_CHECK(top > 0 && top <= ROUTE_MAX_TOP && top <= keep_groups * (E / n_groups),
             "route_scores: the %d largest of %d groups of %d (at most %d)", top, keep_groups, E / n_groups, ROUTE_MAX_TOP);
-  route_scores_kernel<<<(n_tokens + 3) / 4, 256, 0, stream>>>(logits, correction, ids, weights, n_tokens, E, top, n_groups,
-                                                             keep_groups, renorm);
+  route_scores_kernel<<<(n_tokens + 3) / 4, 256, 0, stream>>>(logits, correction, ids, weights, n_tokens, E, ld, top, n_groups,
+                                                             keep_groups, renorm, scale);
   SYN_LAUNCH_CHECK("route_scores");
   return 0;
 }

@@ -822,22 +822,24 @@ def _check_window_pages(k_pages, v_pages, dtype, nkv, dim, vdim, name, v_share=1
 
 
 def window_intake(proj, bias, q_out, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps,
-                  n_heads, n_kv_heads, dim, vdim, write_kv=True, rotation=None, v_share=1):
+                  n_heads, n_kv_heads, dim, vdim, write_kv=True, rotation=None, v_share=1, pairs=False):
     """proj [N, width] float: the fused projection [q | k | v | ...]; bias float [>= q, k, v columns] or None.  q and k
     heads get their bias and (with gains, float [dim]) an RMSNorm over the head; q goes to q_out [N, nh * dim], k and v
     (with its bias) into the pages of sequence tok_seq[n] at position tok_pos[n].
     rotation = (cos, sin) float [positions, rot / 2]: the first `rot` values of every q and k head are then turned by
     the angles of the token's position, value i paired with value i + rot / 2 (the caller sees to it that the tables
-    reach the step's last position).  v_share: there are nkv / v_share value heads (and rows of v in proj)."""
+    reach the step's last position); with `pairs` value 2 i is paired with value 2 i + 1.  v_share: there are
+    nkv / v_share value heads (and rows of v in proj).  write_kv False: the pages are another layer's and are left
+    alone; proj and bias then need to hold the queries only."""
     nh, nkv = n_heads, n_kv_heads
     _need(proj, "window_intake.proj", _F32, (None, None))
     N, width = proj.shape
     if v_share < 1 or nkv % v_share:
         raise KernelError(f"window_intake: {nkv} kv heads in shares of {v_share} value heads")
     nv = nkv // v_share
-    used = (nh + nkv) * dim + nv * vdim
+    used = (nh + nkv) * dim + nv * vdim if write_kv else nh * dim
     if width < used:
-        raise KernelError(f"window_intake: rows of {width} values do not hold q, k and v ({used})")
+        raise KernelError(f"window_intake: rows of {width} values do not hold {'q, k and v' if write_kv else 'q'} ({used})")
     if bias is not None:
         _need(bias, "window_intake.bias", _F32, (None,))
         if bias.shape[0] < used:
@@ -863,19 +865,21 @@ def window_intake(proj, bias, q_out, k_pages, v_pages, page_table, tok_seq, tok_
         _need(k_gain, "window_intake.k_gain", _F32, (dim,))
     _call(load_library("core"), "syn_window_intake", _ptr(proj), width, _ptr(bias), _ptr(q_out), _ptr(k_pages),
           _ptr(v_pages), _is_f32(q_out), _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos),
-          _ptr(q_gain), _ptr(k_gain), ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, N, nh, nkv, nv, dim, vdim,
-          1 if write_kv else 0, _stream())
+          _ptr(q_gain), _ptr(k_gain), ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, 1 if pairs else 0, N, nh, nkv, nv,
+          dim, vdim, 1 if write_kv else 0, _stream())
 
 
 def window_attention(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, n_heads, n_kv_heads, dim, vdim,
                      window=0, keep_first=0, sink_one=False, slopes=None, log_bias=None, softcap=0.0, gate=None,
-                     gate_bias=None, v_share=1):
+                     gate_bias=None, v_share=1, sinks=None, chunk=0, gate_per_head=False):
     """v_share: that many neighbouring kv heads read the values of one value head (v_pages holds nkv / v_share heads).
     Attention of every token (prompts and single tokens alike) whose query is q [N, nh * dim] over the pages
     (which already hold the tokens): score = scale q.k [soft cap] - slopes[h] (i - j) - r1[h] ln(1 + r2[h] (i - j))
     with log_bias = (r1, r2) float [nh]; key j is seen by i iff j <= i and (no window or i - j < window or
-    j < keep_first); sink_one: one more in the softmax's denominator; gate: a float view [N, >= nh * vdim] with row
-    stride gate.stride(0) whose sigmoid multiplies the result; out [N, nh * vdim] in q's type."""
+    j < keep_first) and (no chunk or j // chunk == i // chunk or j < keep_first); sink_one: one more in the softmax's
+    denominator; sinks float [nh]: exp(sinks[h]) more (a learned score of a key without a value); gate: a float view
+    [N, >= nh * vdim] (with gate_per_head [N, >= nh]: one number a head) with row stride gate.stride(0) whose sigmoid
+    multiplies the result; out [N, nh * vdim] in q's type."""
     nh, nkv = n_heads, n_kv_heads
     _need(q, "window_attention.q", (_BF16, _F32), (None, nh * dim))
     N = q.shape[0]
@@ -894,15 +898,26 @@ def window_attention(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, sca
     if slopes is not None:
         _need(slopes, "window_attention.slopes", _F32, (nh,))
     gate_stride = 0
+    n_gate = nh if gate_per_head else nh * vdim
     if gate is not None:
-        gate_stride = _float_rows_view(gate, "window_attention.gate", N, nh * vdim)
+        gate_stride = _float_rows_view(gate, "window_attention.gate", N, n_gate)
         if gate_bias is not None:
-            _need(gate_bias, "window_attention.gate_bias", _F32, (nh * vdim,))
+            _need(gate_bias, "window_attention.gate_bias", _F32, (n_gate,))
+    _sink_and_chunk("window_attention", sinks, sink_one, chunk, nh)
     _call(load_library("core"), "syn_window_attention", _ptr(q), _ptr(k_pages), _ptr(v_pages), _is_f32(q),
           _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos), _ptr(gate), gate_stride,
           _ptr(gate_bias if gate is not None else None), _ptr(out), ctypes.c_float(scale), N, nh, nkv, dim, vdim,
           _ptr(slopes), _ptr(r1), _ptr(r2), ctypes.c_float(float(softcap or 0.0)), int(window or 0), int(keep_first or 0),
-          1 if sink_one else 0, int(v_share), _stream())
+          1 if sink_one else 0, int(v_share), _ptr(sinks), int(chunk or 0), 1 if gate_per_head else 0, _stream())
+
+
+def _sink_and_chunk(name, sinks, sink_one, chunk, n_heads):
+    if sinks is not None:
+        _need(sinks, name + ".sinks", _F32, (n_heads,))
+        if sink_one:
+            raise KernelError(f"{name}: a learned sink and a sink of one together")
+    if chunk is not None and chunk < 0:
+        raise KernelError(f"{name}: chunks of {chunk} positions")
 
 
 WINDOW_PREFILL_MAX_DIM = 128
@@ -915,7 +930,8 @@ def window_prefill_takes(dim, vdim) -> bool:
 
 def window_attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past, out, scale, n_heads, n_kv_heads,
                                   dim, vdim, window=0, keep_first=0, sink_one=False, slopes=None, log_bias=None,
-                                  softcap=0.0, gate=None, gate_bias=None, v_share=1):
+                                  softcap=0.0, gate=None, gate_bias=None, v_share=1, sinks=None, chunk=0,
+                                  gate_per_head=False):
     """window_attention for the new tokens of each sequence of a step in bf16, on the matrix cores: seq_start [B + 1]
     offsets of the sequences' new tokens in q, seq_past [B] tokens cached before (the pages already hold the new
     ones).  Scores and weights are 32-bit; a weight meets V as two bf16 numbers (16 bits of mantissa)."""
@@ -940,15 +956,17 @@ def window_attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, se
     if slopes is not None:
         _need(slopes, "window_attention_prefill.slopes", _F32, (nh,))
     gate_stride = 0
+    n_gate = nh if gate_per_head else nh * vdim
     if gate is not None:
-        gate_stride = _float_rows_view(gate, "window_attention_prefill.gate", N, nh * vdim)
+        gate_stride = _float_rows_view(gate, "window_attention_prefill.gate", N, n_gate)
         if gate_bias is not None:
-            _need(gate_bias, "window_attention_prefill.gate_bias", _F32, (nh * vdim,))
+            _need(gate_bias, "window_attention_prefill.gate_bias", _F32, (n_gate,))
+    _sink_and_chunk("window_attention_prefill", sinks, sink_one, chunk, nh)
     _call(load_library("core"), "syn_window_attention_prefill_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages),
           _ptr(page_table), page_table.shape[1], _ptr(seq_start), _ptr(seq_past), B, N, _ptr(gate), gate_stride,
           _ptr(gate_bias if gate is not None else None), _ptr(out), ctypes.c_float(scale), nh, nkv, dim, vdim,
           _ptr(slopes), _ptr(r1), _ptr(r2), ctypes.c_float(float(softcap or 0.0)), int(window or 0), int(keep_first or 0),
-          1 if sink_one else 0, int(v_share), _stream())
+          1 if sink_one else 0, int(v_share), _ptr(sinks), int(chunk or 0), 1 if gate_per_head else 0, _stream())
 
 
 def _float_rows_view(t, name, n_rows, n_cols):
@@ -1209,20 +1227,25 @@ def measure_ceilings(device="cuda:0", read_bytes=1 << 30, repeats=5):
 def add_scaled_rmsnorm(resid, terms, gain, eps, out, rows=None):
     """resid += sum_t scale_t * delta_t for up to two terms (delta float [N, H] or partial sums [S, N, H], scale float
     [H] or None), then out = RMSNorm(resid) * gain when `out` is given.  rows [n] int32: only those rows are summed and
-    normed, resid is not written."""
+    normed, resid is not written.  A term may be a triple (delta, scale, row_gate): row_gate a float view [N, 1] (a
+    column of longer rows) whose sigmoid multiplies the term's rows."""
     _need(resid, "add_scaled_rmsnorm.resid", _F32, (None, None))
     N, H = resid.shape
     if not 1 <= len(terms) <= 2:
         raise KernelError(f"add_scaled_rmsnorm: {len(terms)} terms (one or two)")
-    args = []
-    for i, (d, s) in enumerate(terms):
+    args, gates = [], []
+    for i, term in enumerate(terms):
+        d, s = term[0], term[1]
+        g = term[2] if len(term) > 2 else None
         parts = d.shape[0] if d.dim() == 3 else 1
         _need(d, f"add_scaled_rmsnorm.delta{i}", _F32, (parts, N, H) if d.dim() == 3 else (N, H))
         if s is not None:
             _need(s, f"add_scaled_rmsnorm.scale{i}", _F32, (H,))
         args += [_ptr(d), parts, _ptr(s)]
+        gates += [_ptr(g), 0 if g is None else _float_rows_view(g, f"add_scaled_rmsnorm.row_gate{i}", N, 1)]
     if len(terms) == 1:
         args += [_ptr(None), 1, _ptr(None)]
+        gates += [_ptr(None), 0]
     n_out = N
     if rows is not None:
         _need(rows, "add_scaled_rmsnorm.rows", _I32, (None,))
@@ -1232,7 +1255,7 @@ def add_scaled_rmsnorm(resid, terms, gain, eps, out, rows=None):
         _need(out, "add_scaled_rmsnorm.out", (_BF16, _F32), (n_out, H))
     elif rows is not None:
         raise KernelError("add_scaled_rmsnorm: gathered rows without an output")
-    _call(load_library("core"), "syn_add_scaled_rmsnorm", _ptr(resid), N, _ptr(rows), n_out, *args, _ptr(gain),
+    _call(load_library("core"), "syn_add_scaled_rmsnorm", _ptr(resid), N, _ptr(rows), n_out, *args, *gates, _ptr(gain),
           0 if gain is None else _is_f32(gain), ctypes.c_float(eps), _ptr(out), 0 if out is None else _is_f32(out), H,
           _stream())
 
@@ -1310,12 +1333,16 @@ def route_sort(ids, weights, n_experts):
     return seg, lists[0], lists[1], lists[2], weight_of
 
 
-def route_scores(logits, correction, ids, weights, n_groups=1, keep_groups=1, renorm=False):
+def route_scores(logits, correction, ids, weights, n_groups=1, keep_groups=1, renorm=False, scale=1.0):
     """A router that scores every expert: s = softmax(logits [N, E] float) over all E; the choice is made on
     s + correction [E] among the members of the keep_groups best of n_groups equal groups of neighbours (a group's
     score: its largest choice score); ids [N, top] int32 the chosen (largest first, the lower index of equal ones),
-    weights [N, top] float their s, divided by their sum with renorm."""
-    _need(logits, "route_scores.logits", _F32, (None, None))
+    weights [N, top] float their s, divided by their sum with renorm, times `scale`.  logits may be the first columns of
+    longer rows (a view with a row stride)."""
+    if isinstance(logits, torch.Tensor) and logits.dim() == 2:
+        ld = _float_rows_view(logits, "route_scores.logits", logits.shape[0], logits.shape[1])
+    else:
+        raise KernelError("route_scores.logits: expected a float matrix on the GPU")
     N, E = logits.shape
     if correction is not None:
         _need(correction, "route_scores.correction", _F32, (E,))
@@ -1326,8 +1353,8 @@ def route_scores(logits, correction, ids, weights, n_groups=1, keep_groups=1, re
         raise KernelError(f"route_scores: {E} experts (at most {ROUTE_MAX_EXPERTS}) in {n_groups} groups, {keep_groups} kept")
     if not 0 < top <= min(keep_groups * (E // n_groups), ROUTE_MAX_TOP):
         raise KernelError(f"route_scores: the {top} largest of {keep_groups} groups of {E // n_groups} (at most {ROUTE_MAX_TOP})")
-    _call(load_library("core"), "syn_route_scores", _ptr(logits), _ptr(correction), _ptr(ids), _ptr(weights), N, E, top,
-          int(n_groups), int(keep_groups), 1 if renorm else 0, _stream())
+    _call(load_library("core"), "syn_route_scores", _ptr(logits), _ptr(correction), _ptr(ids), _ptr(weights), N, E, ld, top,
+          int(n_groups), int(keep_groups), 1 if renorm else 0, ctypes.c_float(float(scale)), _stream())
 
 
 def route_identity(x, out, seg, first, last, a_rows, o_rows, weight_of):

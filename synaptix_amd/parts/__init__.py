@@ -1,6 +1,7 @@
 from .base import Part, KvNeed, StateNeed, flat_needs
 from .norm import RmsNorm, DynamicTanh
-from .position import Position, NoPosition, RotaryHalfSplit, RotaryInterleaved, LogDistanceBias, RotaryScaledHalfSplit
+from .position import (Position, NoPosition, RotaryHalfSplit, RotaryInterleaved, LogDistanceBias, RotaryScaledHalfSplit,
+                       RotaryByWavelength)
 from .mixer import Mixer, GqaAttention, GatedWindowAttention, ParallelMixers, DifferentialAttention
 from .memory import MatrixMemory
 from .recurrent import StateSpaceMixer, ChannelDeltaMixer
@@ -14,4 +15,4 @@ __all__ = ["Part", "KvNeed", "StateNeed", "flat_needs", "RmsNorm", "DynamicTanh"
            "RotaryHalfSplit", "RotaryInterleaved", "LogDistanceBias", "Mixer", "GqaAttention", "GatedWindowAttention", "ParallelMixers",
            "MatrixMemory", "LatentAttention", "FeedForward", "GatedMlp", "RoutedExperts", "Block", "PreNormBlock",
            "HyperConnectionBlock", "ParallelBlock", "linear", "Matrix", "WeightedDeltas", "ChannelScaledDeltas", "SummedDeltas", "RotaryScaledHalfSplit",
-           "DifferentialAttention", "StateSpaceMixer", "ChannelDeltaMixer"]
+           "DifferentialAttention", "StateSpaceMixer", "ChannelDeltaMixer", "RotaryByWavelength"]

@@ -79,8 +79,9 @@ class PreNormBlock(Block):
         from .linear import ChannelScaledDeltas, SummedDeltas
         if scale is None:
             return delta
-        terms = delta.terms if isinstance(delta, SummedDeltas) else [delta]
-        return ChannelScaledDeltas([(t, scale) for t in terms])
+        if isinstance(delta, SummedDeltas):
+            return delta.scaled(scale)
+        return ChannelScaledDeltas([(delta, scale)])
 
     def forward(self, resid, pending, ctx, cache, owner=True):
         # a norm may hand on rows whose last step a product finishes, and take a product that has not been run

@@ -80,13 +80,15 @@ class RoutedExperts(FeedForward):
         "top_logits"  the `top` largest z + bias; weights: softmax over the chosen logits only
         "scores"      s = softmax(z) over all router outputs; the choice is made on s + correction among the members of
                       the `keep_groups` best of `n_groups` equal groups of neighbours (a group's score: its largest choice
-                      score); weights: the chosen s themselves (`renorm`: divided by their sum)
+                      score); weights: the chosen s themselves (`renorm`: divided by their sum) times `route_scale`
     The experts, one of
         ungated       W_down act(W_up h), act the exact GELU
         gated         W_down act2(W_gate h, W_up h) with an activation of the gated products (ops.ACTIVATIONS; one with a
                       bound as the pair (name, bound))
     `identity`: the router's last `identity` outputs stand for experts without tensors whose result is h itself.
-    `shared`: a feed-forward that every token passes as well (its result is a second term of the sum).
+    `shared`: a feed-forward that every token passes as well (its result is a second term of the sum); with
+    `shared_gate` that term is multiplied by sigmoid(w_sg . h), one number a token (tensor `shared_gate` [1, hidden],
+    which rides along as one more row of the router's product).
 
     The tokens are sorted by expert on the device (no count comes back to the host), and each expert's rows meet its
     matrices in one launch for all experts (ops.experts_product).  Returns the `top` weighted results of every token
@@ -102,7 +104,8 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, prefix: str, hidden: int, ff: int, n_experts: int, top: int, activation="gelu",
                  router_bias: bool = True, names=None, *, gated: bool = False, router: str = "top_logits",
-                 n_groups: int = 1, keep_groups: int = 1, renorm: bool = False, identity: int = 0, shared=None):
+                 n_groups: int = 1, keep_groups: int = 1, renorm: bool = False, identity: int = 0, shared=None,
+                 route_scale: float = 1.0, shared_gate: str | None = None):
         if router not in self.ROUTERS:
             raise ValueError(f"{prefix}: router {router!r} (one of {self.ROUTERS})")
         if gated:
@@ -120,6 +123,11 @@ class RoutedExperts(FeedForward):
             raise ValueError(f"{prefix}: {total} router outputs in {n_groups} groups, {keep_groups} kept, {top} chosen")
         if identity and router != "scores":
             raise ValueError(f"{prefix}: identity experts come with the router that scores all outputs")
+        if route_scale != 1.0 and router != "scores":
+            raise ValueError(f"{prefix}: a factor on the weights comes with the router that scores all outputs")
+        if shared_gate is not None and shared is None:
+            raise ValueError(f"{prefix}: a gate for a shared expert that is not there")
+        self.route_scale, self.shared_gate = float(route_scale), shared_gate
         self.prefix, self.hidden, self.ff, self.n_experts, self.top = prefix, hidden, ff, n_experts, top
         self.activation, self.gated, self.router = activation, bool(gated), router
         self.n_groups, self.keep_groups, self.renorm, self.identity = int(n_groups), int(keep_groups), bool(renorm), int(identity)
@@ -146,6 +154,8 @@ class RoutedExperts(FeedForward):
             specs[p + down.format(e)] = TensorSpec((self.hidden, self.ff))
         if self.shared is not None:
             specs.update(self.shared.tensor_specs())
+        if self.shared_gate is not None:
+            specs[p + self.shared_gate] = TensorSpec((1, self.hidden))
         return specs
 
     def load(self, get):
@@ -163,7 +173,10 @@ class RoutedExperts(FeedForward):
             w_down = torch.stack([get(p + down.format(e)) for e in range(self.n_experts)]).contiguous()
             packed = ops.pack_expert_weights(w_down)
             self.w_down = w_down if packed is None else packed
-        self.w_router = Matrix(get(p + router))
+        rows = get(p + router)
+        if self.shared_gate is not None:       # the shared expert's gate as the router's last row
+            rows = torch.cat([rows, get(p + self.shared_gate).to(rows.dtype)], 0)
+        self.w_router = Matrix(rows)
         self.b_router = get(p + bias).float().contiguous() if self.router_bias else None
         if self.shared is not None:
             self.shared.load(get)
@@ -181,10 +194,14 @@ class RoutedExperts(FeedForward):
         ids = torch.empty((N, self.top), dtype=torch.int32, device=dev)
         weights = torch.empty((N, self.top), dtype=torch.float32, device=dev)
         logits = linear(h, self.w_router, torch.float32)
+        shared_gate = None
+        if self.shared_gate is not None:
+            logits, shared_gate = logits[:, :self.total], logits[:, self.total:]
         if self.router == "scores":
-            ops.route_scores(logits, self.b_router, ids, weights, self.n_groups, self.keep_groups, self.renorm)
+            ops.route_scores(logits, self.b_router, ids, weights, self.n_groups, self.keep_groups, self.renorm,
+                             self.route_scale)
         else:
-            ops.route_topk(logits, self.b_router, ids, weights)
+            ops.route_topk(logits.contiguous(), self.b_router, ids, weights)
         seg, tok_of, pair_of, part_of, weight_of = ops.route_sort(ids, weights, self.total)
         y = torch.empty((self.top, N, self.hidden), dtype=torch.float32, device=dev)
         if self.n_experts:
@@ -201,5 +218,5 @@ class RoutedExperts(FeedForward):
                                weight_of)
         if self.shared is not None:
             from .linear import SummedDeltas
-            return SummedDeltas([y, self.shared.forward(h, ctx)])
+            return SummedDeltas([y, self.shared.forward(h, ctx)], [None, shared_gate])
         return y

@@ -126,11 +126,13 @@ class StreamsWrite:
 class ChannelScaledDeltas:
     """The results of one or two sublayers that ran side by side, not yet added to the residual:
     sum_i scale_i * term_i, each term a float tensor [N, hidden] or partial sums [P, N, hidden], each scale float
-    [hidden] (one factor for every channel) or None.  A norm that takes it (RmsNorm) adds the terms into the residual
-    and norms the rows in the same pass; everything else asks for `run()`, the sum as one tensor."""
+    [hidden] (one factor for every channel) or None.  A term may be a triple whose third member is a gate for every row
+    (a float view [N, 1], a column of longer rows, or None): the term then counts sigmoid(gate) times.  A norm that
+    takes it (RmsNorm) adds the terms into the residual and norms the rows in the same pass; everything else asks for
+    `run()`, the sum as one tensor."""
 
     def __init__(self, terms):
-        self.terms = [(as_delta(t), s) for t, s in terms]
+        self.terms = [(as_delta(t[0]), t[1], t[2] if len(t) > 2 else None) for t in terms]
         self.shape = tuple(self.terms[0][0].shape[-2:])
 
     def run(self):
@@ -142,16 +144,25 @@ class ChannelScaledDeltas:
 
 class SummedDeltas:
     """A sublayer's result as several terms that have not been added yet (routed experts and an expert that every token
-    passes), each a float tensor [N, hidden] or partial sums [P, N, hidden] (or a product that has not been run).  A
-    block that scales its sublayers' results by channel hands the terms on, each with the scales
-    (ChannelScaledDeltas); everything else asks for `run()`, the sum as one tensor."""
+    passes), each a float tensor [N, hidden] or partial sums [P, N, hidden] (or a product that has not been run).
+    `row_gates`: for each term None or a float view [N, 1] whose sigmoid multiplies the term's rows (an expert that
+    every token passes through a gate of its own).  A block that scales its sublayers' results by channel hands the
+    terms on, each with the scales; a norm takes them as they are (both as ChannelScaledDeltas); everything else asks
+    for `run()`, the sum as one tensor."""
 
-    def __init__(self, terms):
+    def __init__(self, terms, row_gates=None):
         self.terms = [as_delta(t) for t in terms]
+        self.row_gates = list(row_gates) if row_gates is not None else [None] * len(self.terms)
+        if len(self.row_gates) != len(self.terms):
+            raise ValueError("one gate (or None) for each term")
         self.shape = tuple(self.terms[0].shape[-2:])
 
+    def scaled(self, scale=None):
+        """The terms, each with the channels' scales `scale` (or none) and its rows' gate."""
+        return ChannelScaledDeltas([(t, scale, g) for t, g in zip(self.terms, self.row_gates)])
+
     def run(self):
-        return ChannelScaledDeltas([(t, None) for t in self.terms]).run()
+        return self.scaled().run()
 
 
 def as_delta(d):

@@ -187,57 +187,93 @@ class GatedWindowAttention(Mixer):
 
         score(i, j) = scale q_i.k_j [soft cap] + what the position scheme puts on the scores
         key j is seen by i iff j <= i and (window is None or i - j < window or j < keep_first)
-        p_j = exp(score_j) / (sink + sum exp(score_j)),  sink = 1 with sink_one
+                                      and (chunk is None or j // chunk == i // chunk or j < keep_first)
+        p_j = exp(score_j) / (sink + sum exp(score_j)),  sink = 1 with sink_one, exp(sink_h) with a learned `sink`
 
     Keys have `dim` values, values `v_dim`.  q, k and v may carry a bias (`bias`), the output product one of its own
     (`out_bias`); q and k heads may be normed (RMS over the head, one gain for all heads: `qk_norm_eps`); with `gate`
-    the heads' results are multiplied by sigmoid(W_g h) before the output product.  The position scheme may rotate
-    nothing here: it acts on the scores (Position.score_slopes, Position.score_log_bias).  Scores, weights and the
-    norms are 32-bit in both engine types.
+    the heads' results are multiplied by sigmoid(W_g h) before the output product (True or "value": one gate for every
+    value; "head": one for each head).  The position scheme may act on the scores (Position.score_slopes,
+    Position.score_log_bias) or turn the first values of every q and k head after the norm (Position.tables, in the
+    pairing that Position.pairing names).  `chunk`: positions are counted in runs of that many from the sequence's
+    first token, and a query sees the keys of its own run only.  Scores, weights, the rotation and the norms are 32-bit
+    in both engine types.
 
-    Tensor names: prefix + "q", "k", "v", "o" (+ ".b" for their biases), "q.norm", "k.norm", "g"; `names` renames them.
+    `shared_kv`: the layer has no keys and values of its own (no k and v tensors, biases or k norm): it reads the cache
+    of an earlier layer with the same head counts and sizes (the model's schedule gives both runs the same cache), as
+    that layer wrote it, with its own queries, mask, sink and gate.  `cache_window`: what the cache keeps where that is
+    more than this layer's own mask needs (the layers that share a cache name the same).
+
+    Tensor names: prefix + "q", "k", "v", "o" (+ ".b" for their biases), "q.norm", "k.norm", "g", "sink"; `names`
+    renames them.
     """
     takes_scaled_rows = False
     capturable = True
 
-    NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "g": "g", "q_norm": "q.norm", "k_norm": "k.norm", "bias": ".b"}
+    NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "g": "g", "q_norm": "q.norm", "k_norm": "k.norm", "bias": ".b",
+             "sink": "sink"}
+    _UNSET = object()
 
     def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, dim: int, v_dim: int | None = None, *,
                  position: Position | None = None, qk_norm_eps: float | None = None, scale: float | None = None,
                  window: int | None = None, keep_first: int = 0, sink_one: bool = False, bias: bool = False,
-                 out_bias: bool = False, gate: bool = False, score_softcap: float | None = None, names: dict | None = None):
+                 out_bias: bool = False, gate=False, score_softcap: float | None = None, names: dict | None = None,
+                 chunk: int | None = None, sink: bool = False, shared_kv: bool = False, cache_window=_UNSET):
         if n_kv_heads <= 0 or n_heads % n_kv_heads:
             raise ValueError(f"{n_heads} heads do not divide into {n_kv_heads} kv heads")
+        if gate not in (False, True, None, "value", "head"):
+            raise ValueError(f"{prefix}: gate {gate!r} (False, 'value' or 'head')")
+        if sink and sink_one:
+            raise ValueError(f"{prefix}: a learned sink and a sink of one together")
+        if chunk is not None and chunk <= 0:
+            raise ValueError(f"{prefix}: chunks of {chunk} positions")
         self.prefix, self.hidden = prefix, hidden
         self.nh, self.nkv, self.dim, self.vdim = n_heads, n_kv_heads, dim, v_dim or dim
         self.position = position or NoPosition()
         self.qk_norm_eps = qk_norm_eps
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(dim)
         self.window, self.keep_first, self.sink_one = window, int(keep_first or 0), bool(sink_one)
-        self.bias, self.out_bias, self.gate = bool(bias), bool(out_bias), bool(gate)
+        self.chunk, self.sink, self.shared_kv = chunk, bool(sink), bool(shared_kv)
+        # what a query can see lies within the last `reach` positions (None: anywhere): a run of `chunk` positions is
+        # never longer than that many
+        reach = [n for n in (window, chunk) if n]
+        self.reach = min(reach) if reach else None
+        self.cache_window = self.reach if cache_window is self._UNSET else cache_window
+        if self.cache_window is not None and (self.reach is None or self.cache_window < self.reach):
+            raise ValueError(f"{prefix}: a cache of the last {self.cache_window} keys for a mask that reaches "
+                             f"{'every key' if self.reach is None else self.reach}")
+        self.bias, self.out_bias = bool(bias), bool(out_bias)
+        self.gate = "head" if gate == "head" else ("value" if gate else None)
         self.score_softcap = float(score_softcap) if score_softcap else 0.0
         self.names = dict(self.NAMES, **(names or {}))
-        self.w_in = self.w_o = self.b_in = self.b_o = self.q_gain = self.k_gain = None
+        self.w_in = self.w_o = self.b_in = self.b_o = self.q_gain = self.k_gain = self.sinks = None
         self._terms = None
 
     def _n(self, key, bias=False):
         return self.prefix + self.names[key] + (self.names["bias"] if bias else "")
 
+    def _biased(self):
+        """The pieces of the fused projection that carry a bias: q, and k and v where the layer has them."""
+        return [("q", self.nh * self.dim)] + ([] if self.shared_kv else [("k", self.nkv * self.dim), ("v", self.nkv * self.vdim)])
+
     def _widths(self):
-        return [("q", self.nh * self.dim), ("k", self.nkv * self.dim), ("v", self.nkv * self.vdim)] + \
-               ([("g", self.nh * self.vdim)] if self.gate else [])
+        gate = {None: 0, "head": self.nh, "value": self.nh * self.vdim}[self.gate]
+        return self._biased() + ([("g", gate)] if self.gate else [])
 
     def tensor_specs(self):
         specs = {self._n(k): TensorSpec((n, self.hidden)) for k, n in self._widths()}
         specs[self._n("o")] = TensorSpec((self.hidden, self.nh * self.vdim))
         if self.bias:
-            for k, n in self._widths()[:3]:
+            for k, n in self._biased():
                 specs[self._n(k, True)] = TensorSpec((n,), "bias")
         if self.out_bias:
             specs[self._n("o", True)] = TensorSpec((self.hidden,), "bias")
         if self.qk_norm_eps is not None:
             specs[self._n("q_norm")] = TensorSpec((self.dim,), "gain")
-            specs[self._n("k_norm")] = TensorSpec((self.dim,), "gain")
+            if not self.shared_kv:
+                specs[self._n("k_norm")] = TensorSpec((self.dim,), "gain")
+        if self.sink:
+            specs[self._n("sink")] = TensorSpec((self.nh,), "bias")
         specs.update(self.position.tensor_specs())
         return specs
 
@@ -246,23 +282,27 @@ class GatedWindowAttention(Mixer):
         self.w_in = _projection(torch.cat([get(self._n(k)) for k, _ in self._widths()], 0))
         self.w_o = _projection(get(self._n("o")))
         if self.bias:
-            self.b_in = torch.cat([get(self._n(k, True)).float() for k, _ in self._widths()[:3]]).contiguous()
+            self.b_in = torch.cat([get(self._n(k, True)).float() for k, _ in self._biased()]).contiguous()
         if self.out_bias:
             self.b_o = get(self._n("o", True)).float().contiguous()
         if self.qk_norm_eps is not None:
             self.q_gain = get(self._n("q_norm")).float().contiguous()
-            self.k_gain = get(self._n("k_norm")).float().contiguous()
+            # (a layer without keys of its own hands the intake its query gain twice; the key gain is never read)
+            self.k_gain = self.q_gain if self.shared_kv else get(self._n("k_norm")).float().contiguous()
+        if self.sink:
+            self.sinks = get(self._n("sink")).float().contiguous()
         self.position.load(get)
 
     def cache_need(self):
-        return KvNeed(self.nkv, self.dim, self.window, v_dim=self.vdim, keep_first=self.keep_first if self.window else 0)
+        return KvNeed(self.nkv, self.dim, self.cache_window, v_dim=self.vdim,
+                      keep_first=self.keep_first if self.cache_window else 0)
 
     def check(self, dtype):
         if max(self.dim, self.vdim) > ops.WINDOW_ATTENTION_MAX_DIM:
             raise ValueError(f"{self.prefix}: head sizes {self.dim} and {self.vdim} (at most {ops.WINDOW_ATTENTION_MAX_DIM})")
         cos, _ = self.position.tables("cpu")
-        if cos is not None:
-            raise ValueError(f"{self.prefix}: this attention takes position schemes that act on the scores, not rotations")
+        if cos is not None and 2 * cos.shape[1] > self.dim:
+            raise ValueError(f"{self.prefix}: the rotation turns {2 * cos.shape[1]} values of heads of {self.dim}")
 
     def _score_terms(self, device):
         if self._terms is None:
@@ -273,15 +313,22 @@ class GatedWindowAttention(Mixer):
 
     def forward(self, h, ctx, cache, owner=True):
         N, act = h.shape[0], h.dtype
-        proj = linear(h, self.w_in, torch.float32)          # [N, q | k | v | gate] float
+        if owner == self.shared_kv:
+            raise ValueError(f"{self.prefix}: a layer {'without' if owner else 'with'} keys and values of its own was "
+                             f"scheduled as the cache's {'owner' if owner else 'reader'}")
+        cap = self.position.capacity
+        if cap is not None and ctx.max_position >= cap:
+            raise ValueError(f"position {ctx.max_position} is beyond the position encoding's capacity {cap}")
+        proj = linear(h, self.w_in, torch.float32)          # [N, q | k | v | gate] float (q | gate with shared_kv)
         q = torch.empty((N, self.nh * self.dim), dtype=act, device=h.device)
         table = ctx.page_table(cache.group)
         ops.window_intake(proj, self.b_in, q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos,
                           self.q_gain, self.k_gain, self.qk_norm_eps or 0.0, self.nh, self.nkv, self.dim, self.vdim,
-                          write_kv=owner)
+                          write_kv=owner, rotation=self.position.tables(h.device), pairs=self.position.pairing == "pairs")
         o = torch.empty((N, self.nh * self.vdim), dtype=act, device=h.device)
-        gate = proj[:, (self.nh + self.nkv) * self.dim + self.nkv * self.vdim:] if self.gate else None
+        gate = proj[:, sum(n for _, n in self._biased()):] if self.gate else None
         how = dict(window=self.window or 0, keep_first=self.keep_first, sink_one=self.sink_one, gate=gate,
+                   gate_per_head=self.gate == "head", sinks=self.sinks, chunk=self.chunk or 0,
                    **self._score_terms(h.device))
         if act == torch.bfloat16 and not ctx.one_token_each and ops.window_prefill_takes(self.dim, self.vdim):
             # prompts in bf16: tiles of queries on the matrix cores

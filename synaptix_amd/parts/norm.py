@@ -13,7 +13,7 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part
-from .linear import DeferredProduct, ScaledRows, ChannelScaledDeltas
+from .linear import DeferredProduct, ScaledRows, ChannelScaledDeltas, SummedDeltas
 
 
 class RmsNorm(Part):
@@ -38,9 +38,12 @@ class RmsNorm(Part):
     def add_apply(self, resid, delta, out_dtype, rows=None):
         """resid [N, dim] float: with rows None, resid += delta (if any) in place and every row is
         normed; with rows [n] int32 only those rows of resid + delta are normed and resid is kept."""
+        if isinstance(delta, SummedDeltas):
+            # a sublayer's result in several terms (routed experts' partial sums, a gated shared expert)
+            delta = delta.scaled() if len(delta.terms) <= 2 else delta.run()
         if isinstance(delta, ChannelScaledDeltas):
             # the results of sublayers that ran side by side, each with its channels' scales: added and normed in one pass
-            if self.gain_offset == 0.0:
+            if self.gain_offset == 0.0 and len(delta.terms) <= 2:
                 n = resid.shape[0] if rows is None else rows.shape[0]
                 out = torch.empty((n, self.dim), dtype=out_dtype, device=resid.device)
                 ops.add_scaled_rmsnorm(resid, delta.terms, self.gain, self.eps, out, rows)

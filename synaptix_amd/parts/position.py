@@ -30,6 +30,8 @@ class Position(Part):
         return None
 
     capacity = None  # positions at and beyond it cannot be encoded; None: no limit
+    # which values a rotation pairs: "halves" (value i with value i + rotary_dim / 2) or "pairs" (value 2i with 2i + 1)
+    pairing = "halves"
 
 
 class NoPosition(Position):
@@ -95,6 +97,7 @@ class RotaryInterleaved(Position):
     passes unchanged.  Tables [capacity, dims / 2] are made on the host with 64-bit angles and kept in 32-bit, once for
     all parts with the same constants."""
     capturable = True
+    pairing = "pairs"
     _shared: dict = {}
 
     def __init__(self, base: float, dims: int, capacity: int):
@@ -171,6 +174,58 @@ class RotaryScaledHalfSplit(Position):
         if self.dims == 0:
             return None, None
         key = (self.base, self.dims, self.capacity, self.factor, self.original, self.fast, self.slow, str(device))
+        if key not in self._shared:
+            cos, sin = self.host_tables()
+            self._shared[key] = (torch.from_numpy(cos).to(device), torch.from_numpy(sin).to(device))
+        return self._shared[key]
+
+
+class RotaryByWavelength(Position):
+    """A rotation of the first `dims` values whose rates depend on their wavelength, for contexts beyond the `original`
+    one that the plain rates f_i = base^(-2i / dims) were made for.  With the wavelength l_i = 2 pi / f_i:
+
+        l_i < original / high:   rate_i = f_i                       (fast waves stay)
+        l_i > original / low:    rate_i = f_i / factor              (slow waves are stretched)
+        else:                    s = (original / l_i - low) / (high - low);  rate_i = (1 - s) f_i / factor + s f_i
+
+    factor None: the plain rates.  pairing "halves" (value i with i + dims / 2) or "pairs" (2i with 2i + 1); the mixer
+    that takes the tables asks for it.  Tables [capacity, dims / 2] from 64-bit angles, kept in 32-bit, once for all parts
+    with the same constants."""
+    capturable = True
+    _shared: dict = {}
+
+    def __init__(self, base: float, dims: int, capacity: int, factor: float | None = None, low: float | None = None,
+                 high: float | None = None, original: float | None = None, pairing: str = "halves"):
+        if dims < 0 or dims % 2:
+            raise ValueError(f"rotated dims {dims} must be even and not negative")
+        if capacity <= 0:
+            raise ValueError("capacity must be positive")
+        if pairing not in ("halves", "pairs"):
+            raise ValueError(f"pairing {pairing!r} ('halves' or 'pairs')")
+        if factor is not None and (low is None or high is None or original is None or not factor > 0.0 or not high > low):
+            raise ValueError("stretched rates need factor, low < high and original")
+        self.base, self.dims, self.capacity, self.pairing = float(base), int(dims), int(capacity), pairing
+        self.factor, self.low, self.high, self.original = factor, low, high, original
+
+    def rates(self):
+        """rate_i as float64 [dims / 2]."""
+        import math
+        f = np.power(np.float64(self.base), -2.0 * np.arange(self.dims // 2, dtype=np.float64) / max(self.dims, 1))
+        if self.factor is None:
+            return f
+        wave = 2.0 * math.pi / f
+        s = (self.original / wave - self.low) / (self.high - self.low)
+        blend = (1.0 - s) * f / self.factor + s * f
+        return np.where(wave < self.original / self.high, f, np.where(wave > self.original / self.low, f / self.factor, blend))
+
+    def host_tables(self):
+        ang = np.arange(self.capacity, dtype=np.float64)[:, None] * self.rates()[None, :]
+        return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+    def tables(self, device):
+        if self.dims == 0:
+            return None, None
+        key = (self.base, self.dims, self.capacity, self.factor, self.low, self.high, self.original, str(device))
         if key not in self._shared:
             cos, sin = self.host_tables()
             self._shared[key] = (torch.from_numpy(cos).to(device), torch.from_numpy(sin).to(device))

@@ -110,7 +110,8 @@ def attention_chunked(h, w, p, c, kv=None):
     q = rotate((h @ w[p + "q"].T).view(T, H, D), f, "pairs")
     k = rotate((h @ w[p + "k"].T).view(T, G, D), f, "pairs")
     v = (h @ w[p + "v"].T).view(T, G, E)
-    o = attend(q, k, v, c["scale"], chunk_mask(T, c["mask"]["size"]), w[p + "sink"])
+    mask = chunk_mask(T, c["mask"]["size"]) if c.get("mask") else window_mask(T, None)
+    o = attend(q, k, v, c["scale"], mask, w[p + "sink"])
     return o.reshape(T, H * E) @ w[p + "o"].T, (k, v)
 
 
@@ -131,7 +132,7 @@ def attention_windowed(h, w, p, c, eps, kv=None):
         v = (h @ w[p + "v"].T + w[p + "v.b"]).view(T, G, E)
     else:
         k, v = kv
-    o = attend(q, k, v, c["scale"], window_mask(T, c["mask"]["size"]), w[p + "sink"])
+    o = attend(q, k, v, c["scale"], window_mask(T, c["mask"]["size"] if c.get("mask") else None), w[p + "sink"])
     o = o * torch.sigmoid(h @ w[p + "g"].T)[:, :, None]
     return o.reshape(T, H * E) @ w[p + "o"].T, (k, v)
 

@@ -2,7 +2,7 @@
 """Throughput of the engine at a Qwen3 shape with random bf16 weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape 8b|4b|32b] [--batch 8] [--layers L]
-    python bench.py --design bizipel|kamivik|repolix [--sizes small,mid,large] [--prompt 2048] [--batch 8] [--window 1024]
+    python bench.py --design bizipel|kamivik|repolix|nilepel [--sizes small,mid,large] [--prompt 2048] [--batch 8] [--window 1024]
 
 --shape 8b (the default) and 32b: a step is one decode step of `batch` sequences, each after a
 2,048-token prompt of uniform ids, run through the same captured graph and host loop that
@@ -32,6 +32,11 @@ token uses `top`, top x the expert's width being the dense feed-forward's width.
 state of 128 rows, 8 groups), delta rule (the heads and head size of the attention), attention in two maps of half the
 head size over shared values with the window, state space; gated experts of which each token uses top - 1 beside one
 shared expert (together the dense feed-forward's width), two identity experts, two groups of which one stays.
+--design nilepel: the same for the Nilepel design: layers in the order windowed attention (biases, q/k norms, half of each
+head turned with stretched long waves, a sink, a gate a head), latent attention (a latent of 512 beside 64 turned values, the
+window), attention over runs of `window` positions (pairs turned, a sink), windowed attention again on the first layer's
+keys and values; the first and third layers with a bounded dense feed-forward, the others with silu experts of which each
+token uses top - 1 within one of two groups beside a gated shared expert (together the dense feed-forward's width).
 
 Method after the reference's own harnesses (crates/synaptix-models/llm/qwen3/examples/format_perf.rs:41-122,
 crates/synaptix-cli/src/commands/bench.rs:35-96): synthetic ids, warm-up first, device synchronised
@@ -183,6 +188,7 @@ SIDE_BY_SIDE_SIZES = {     # layers, width, heads, kv heads, head size, feed-for
 
 KAMIVIK_EXPERTS = {"small": (4, 1024), "mid": (4, 2048), "large": (6, 2048)}      # (top, an expert's width); 8 x top experts
 REPOLIX_ORDER = ("mamba2", "channel_delta", "attention", "mamba2")
+NILEPEL_ORDER = ("attention_2", "latent_attention", "attention", "attention_2")
 
 
 def repolix_experts(size):
@@ -199,7 +205,7 @@ def design_configs(design, size, window, context):
     layers have latent attention (a latent of 512, 64 rotated values, unrotated keys and values of the head size; every
     second layer with the window) and a mixture of experts whose active width equals the dense feed-forward's."""
     from synaptix_amd import Qwen3Config
-    from synaptix_amd.config import BizipelConfig, KamivikConfig, RepolixConfig
+    from synaptix_amd.config import BizipelConfig, KamivikConfig, RepolixConfig, NilepelConfig
     L, W, nh, nkv, hd, ff, V = SIDE_BY_SIDE_SIZES[size]
     qwen = Qwen3Config.from_dict(dict(_COMMON, num_hidden_layers=L, hidden_size=W, num_attention_heads=nh,
                                       num_key_value_heads=nkv, head_dim=hd, intermediate_size=ff, vocab_size=V,
@@ -218,6 +224,25 @@ def design_configs(design, size, window, context):
         rep = RepolixConfig.from_dict({"architecture": "Repolix", "vocab": V, "width": W, "norm": {"eps": 1e-6},
                                        "embedding": {"scale": float(W) ** 0.5}, "middle_rank": hd, "layers": layers})
         return qwen, rep
+    if design == "nilepel":
+        E, _, top, eff = repolix_experts(size)
+        moe = {"kind": "moe", "expert": {"ff": eff}, "shared": {"ff": eff},
+               "router": {"experts": E, "top": top, "scale": 1.5, "groups": {"count": 2, "keep": 1}}}
+        dense = {"kind": "dense", "ff": ff, "limit": 7.0}
+        stretched = {"base": 500000.0, "dims": hd // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+        windowed = {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": window},
+                    "rot": stretched}
+        mixers = [windowed,
+                  {"heads": nh, "dim": hd, "rot_dim": 64, "vdim": hd, "kv_rank": 512, "scale": (hd + 64) ** -0.5,
+                   "mask": {"size": window}, "rot": {"base": 10000.0, "dims": 64}},
+                  {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": window},
+                   "rot": {"base": 10000.0, "dims": hd // 2}},
+                  dict(windowed, kv_from=0)]
+        layers = [{"type": NILEPEL_ORDER[i % 4], "mixer": dict(mixers[i % 4], **({"kv_from": i - 3} if i % 4 == 3 else {})),
+                   "mlp": moe if i % 2 else dense} for i in range(L)]
+        nil = NilepelConfig.from_dict({"architecture": "Nilepel", "vocab": V, "width": W, "norm": {"eps": 1e-6},
+                                       "embedding": {"scale": float(W) ** 0.5}, "layers": layers})
+        return qwen, nil
     if design == "kamivik":
         top, eff = KAMIVIK_EXPERTS[size]
         layers = []
@@ -274,6 +299,12 @@ def designs_side_by_side(args) -> int:
                 total, one = E + I, 3 * 2 * eff * cfg.width
                 touched = E * (1.0 - (1.0 - top / total) ** B)
                 weight_bytes -= int(len(cfg.layers) * (E - touched) * one)
+            if design == "nilepel":
+                # likewise, in the layers that have experts (every second one)
+                E, _, top, eff = repolix_experts(size)
+                one = 3 * 2 * eff * cfg.width
+                touched = E * (1.0 - (1.0 - top / E) ** B)
+                weight_bytes -= int(sum(1 for l in cfg.layers if l.mlp.kind == "moe") * (E - touched) * one)
             g = torch.Generator().manual_seed(0)
             prompt = torch.randint(0, cfg.vocab_size, (P,), generator=g).tolist()
             times = []
@@ -344,7 +375,7 @@ def main() -> int:
                     help="the longest sequence (positions and cache a sequence; the contract's run has 8,192)")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
-    ap.add_argument("--design", default=None, choices=["bizipel", "kamivik", "repolix"],
+    ap.add_argument("--design", default=None, choices=["bizipel", "kamivik", "repolix", "nilepel"],
                     help="another run than the default one: this design beside the Qwen3 decoder at equal layer sizes")
     ap.add_argument("--sizes", default="small,mid,large", help="with --design: which of small, mid, large")
     ap.add_argument("--window", type=int, default=1024, help="with --design: the keys a query of the new design sees")

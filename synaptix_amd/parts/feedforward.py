@@ -174,8 +174,11 @@ class RoutedExperts(FeedForward):
             packed = ops.pack_expert_weights(w_down)
             self.w_down = w_down if packed is None else packed
         rows = get(p + router)
-        if self.shared_gate is not None:       # the shared expert's gate as the router's last row
+        if self.shared_gate is not None:       # the shared expert's gate as one more row behind the router's
             rows = torch.cat([rows, get(p + self.shared_gate).to(rows.dtype)], 0)
+            spare = -rows.shape[0] % 16            # (and rows of zeros up to whole fragments of 16, which nobody reads)
+            if spare and rows.shape[1] % 32 == 0:
+                rows = torch.cat([rows, torch.zeros((spare, rows.shape[1]), dtype=rows.dtype, device=rows.device)], 0)
         self.w_router = Matrix(rows)
         self.b_router = get(p + bias).float().contiguous() if self.router_bias else None
         if self.shared is not None:
@@ -196,7 +199,7 @@ class RoutedExperts(FeedForward):
         logits = linear(h, self.w_router, torch.float32)
         shared_gate = None
         if self.shared_gate is not None:
-            logits, shared_gate = logits[:, :self.total], logits[:, self.total:]
+            logits, shared_gate = logits[:, :self.total], logits[:, self.total:self.total + 1]
         if self.router == "scores":
             ops.route_scores(logits, self.b_router, ids, weights, self.n_groups, self.keep_groups, self.renorm,
                              self.route_scale)

@@ -182,6 +182,16 @@ def _projection(w):
     return Matrix(w, keep_rows=w.shape[1] % 128 != 0)
 
 
+def _whole_fragments(w):
+    """A fused projection whose last piece is a few rows (one gate a head): rows of zeros behind it up to the next
+    multiple of 16, so that the matrix can lie in fragment order; the product's rows get that much longer, and nobody
+    reads the extra columns."""
+    spare = -w.shape[0] % 16
+    if spare == 0 or w.shape[1] % 128:
+        return w
+    return torch.cat([w, torch.zeros((spare, w.shape[1]), dtype=w.dtype, device=w.device)], 0)
+
+
 class GatedWindowAttention(Mixer):
     """Grouped-query attention whose scores, mask and softmax are parameters (csrc/attention_window.hip):
 
@@ -279,7 +289,7 @@ class GatedWindowAttention(Mixer):
 
     def load(self, get):
         # one product for q, k, v and the gate: rows of the matrices one after another
-        self.w_in = _projection(torch.cat([get(self._n(k)) for k, _ in self._widths()], 0))
+        self.w_in = _projection(_whole_fragments(torch.cat([get(self._n(k)) for k, _ in self._widths()], 0)))
         self.w_o = _projection(get(self._n("o")))
         if self.bias:
             self.b_in = torch.cat([get(self._n(k, True)).float() for k, _ in self._biased()]).contiguous()
@@ -326,7 +336,8 @@ class GatedWindowAttention(Mixer):
                           self.q_gain, self.k_gain, self.qk_norm_eps or 0.0, self.nh, self.nkv, self.dim, self.vdim,
                           write_kv=owner, rotation=self.position.tables(h.device), pairs=self.position.pairing == "pairs")
         o = torch.empty((N, self.nh * self.vdim), dtype=act, device=h.device)
-        gate = proj[:, sum(n for _, n in self._biased()):] if self.gate else None
+        at = sum(n for _, n in self._biased())
+        gate = proj[:, at:at + self._widths()[-1][1]] if self.gate else None
         how = dict(window=self.window or 0, keep_first=self.keep_first, sink_one=self.sink_one, gate=gate,
                    gate_per_head=self.gate == "head", sinks=self.sinks, chunk=self.chunk or 0,
                    **self._score_terms(h.device))

@@ -62,14 +62,12 @@ class Rotation:
     scaling: Optional[WavelengthScaling] = None
 
     @classmethod
-    def from_dict(cls, d, where, most, scaling_allowed=False):
+    def from_dict(cls, d, where, most):
         if d.get("rot") is None:
             return cls(10000.0, 0)
         rot, at = _obj(d, "rot", where), where + ".rot"
         scaling = None
         if rot.get("scaling") is not None:
-            if not scaling_allowed:
-                raise ConfigError(f"{at}: 'scaling' is not a key of this mixer")
             scaling = WavelengthScaling.from_dict(_obj(rot, "scaling", at), at + ".scaling")
         c = cls(_num(rot, "base", at), _int(rot, "dims", at, 0), scaling)
         if c.dims % 2 or c.dims > most:
@@ -106,18 +104,21 @@ class ChunkedAttentionConfig:
     chunk: Optional[int]           # mask.size; None: every earlier key
     rot: Rotation
 
-    kv_from = None
+    kv_from: Optional[int] = None  # the layer whose keys and values this one reads; None: its own
 
     @classmethod
     def from_dict(cls, d, where):
         heads, kv = _heads(d, where)
         dim = _int(d, "dim", where)
         return cls(heads, kv, dim, _int(d, "vdim", where), _scale(d, where, dim), _mask(d, where),
-                   Rotation.from_dict(d, where, dim))
+                   Rotation.from_dict(d, where, dim), _int(d, "kv_from", where, 0) if d.get("kv_from") is not None else None)
 
     def to_dict(self):
-        return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale,
-                "rot": self.rot.to_dict(), **_mask_dict(self.chunk)}
+        d = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale,
+             "rot": self.rot.to_dict(), **_mask_dict(self.chunk)}
+        if self.kv_from is not None:
+            d["kv_from"] = self.kv_from
+        return d
 
 
 @dataclass(frozen=True)
@@ -136,7 +137,7 @@ class WindowAttentionConfig:
         heads, kv = _heads(d, where)
         dim = _int(d, "dim", where)
         return cls(heads, kv, dim, _int(d, "vdim", where), _scale(d, where, dim), _mask(d, where),
-                   Rotation.from_dict(d, where, dim, scaling_allowed=True),
+                   Rotation.from_dict(d, where, dim),
                    _int(d, "kv_from", where, 0) if d.get("kv_from") is not None else None)
 
     def to_dict(self):
@@ -286,7 +287,7 @@ class NilepelConfig:
 
     def kv_source(self, i: int) -> int:
         """The layer whose cache layer i reads: itself, or where its chain of `kv_from` ends.  The source runs earlier,
-        is of the same type and has the same head counts and sizes."""
+        keeps keys and values by head, and has the same head counts and sizes."""
         m, at = self.layers[i].mixer, i
         while self.layers[at].mixer.kv_from is not None:
             src = self.layers[at].mixer.kv_from
@@ -294,9 +295,9 @@ class NilepelConfig:
                 raise ConfigError(f"layers[{at}].mixer: kv_from {src} must name an earlier layer")
             at = src
         s = self.layers[at].mixer
-        if at != i and (self.layers[at].type != self.layers[i].type
+        if at != i and (self.layers[at].type == "latent_attention"
                         or (s.heads, s.kv_heads, s.dim, s.vdim) != (m.heads, m.kv_heads, m.dim, m.vdim)):
-            raise ConfigError(f"layers[{i}].mixer: kv_from {at} names a layer of another type or other head sizes")
+            raise ConfigError(f"layers[{i}].mixer: kv_from {at} names a layer of another kind or other head sizes")
         return at
 
     @classmethod

@@ -49,7 +49,8 @@ def _mixer(cfg, i, p, capacity, cache_window):
                                norm_eps=eps, scale=m.scale, window=m.window, gate=None)
     if layer.type == "attention":
         return GatedWindowAttention(p, W, m.heads, m.kv_heads, m.dim, m.vdim, position=_rotation(m.rot, capacity, "pairs"),
-                                    scale=m.scale, chunk=m.chunk, sink=True, cache_window=cache_window)
+                                    scale=m.scale, chunk=m.chunk, sink=True, shared_kv=m.kv_from is not None,
+                                    cache_window=cache_window)
     return GatedWindowAttention(p, W, m.heads, m.kv_heads, m.dim, m.vdim, position=_rotation(m.rot, capacity, "halves"),
                                 qk_norm_eps=eps, scale=m.scale, window=m.window, sink=True, bias=True, gate="head",
                                 shared_kv=m.kv_from is not None, cache_window=cache_window)

@@ -12,11 +12,13 @@ from synaptix_amd import write_random_model
 from plain_nilepel import PlainNilepel
 
 
-def chunked(heads, kv_heads, dim, vdim, chunk=None, dims=None, base=10000.0, scale=None):
+def chunked(heads, kv_heads, dim, vdim, chunk=None, dims=None, base=10000.0, scale=None, kv_from=None):
     m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale if scale is not None else 8.0 * dim ** -0.5,
          "rot": {"base": base, "dims": dim if dims is None else dims}}
     if chunk is not None:
         m["mask"] = {"size": chunk}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
     return "attention", m
 
 
@@ -74,6 +76,8 @@ def config(vocab, width, layers, eps=1e-6, scale=None):
 #    the embedding.
 # R: sizes at which the products run on the matrix cores and prompts' attention in tiles; a window that no test sequence
 #    outgrows; runs of two pages; sixteen experts in four groups; two layers reading one layer's keys.
+# T: a width, feed-forwards and a vocabulary that are multiples of two at most; a layer over runs that reads the keys of a
+#    windowed layer (turned in halves by that layer, its own queries in pairs); an expert layer whose groups all stay.
 # S: one head everywhere, a window of one and of two, runs of one position, the top one of two experts: a choice that the
 #    rounding of bfloat16 activations can turn changes a token's result altogether, so this one is 32-bit only.
 CONFIGS = {
@@ -94,12 +98,15 @@ CONFIGS = {
                            (chunked(4, 4, 32, 64, chunk=128, dims=16), moe(32, 8, 2, shared=64)),
                            (windowed(8, 2, 64, 32, dims=32, scaling=(8.0, 1.0, 2.0, 128), base=1e6, kv_from=2), dense(128, 1.0))],
                 scale=11.3),
+    "T": config(131, 90, [(windowed(5, 5, 6, 14, window=9, dims=6), moe(22, 6, 2, groups=(3, 3), scale=0.5, shared=10)),
+                          (latent(3, 6, 4, 10, 14, window=70), dense(34, 1.2)),
+                          (chunked(5, 5, 6, 14, chunk=40, dims=4, kv_from=0), dense(18, 0.8))], scale=1.7),
     "S": config(101, 40, [(windowed(1, 1, 8, 8, window=1), moe(16, 2, 1)),
                           (chunked(1, 1, 6, 12, chunk=1, dims=2), None),
                           (latent(1, 4, 2, 6, 5, window=2), dense(24, 1.0)),
                           (windowed(1, 1, 8, 8, window=2, kv_from=0), None)], scale=2.0),
 }
-SEEDS = {"P": 41, "Q": 42, "R": 43, "S": 44}
+SEEDS = {"P": 41, "Q": 42, "R": 43, "S": 44, "T": 45}
 
 
 def dtypes_of(name: str) -> list:

@@ -103,13 +103,16 @@ def attend(q, k, v, scale, mask, sink=None):
 # ---------------------------------------------------------------- mixers
 def attention_chunked(h, w, p, c, kv=None):
     """Mixer "attention": no biases, pairs rotated, chunks, a sink.  Returns (delta, (k, v)) with the keys as a later
-    layer would read them."""
+    layer would read them; with kv given it makes queries only."""
     T = h.shape[0]
     H, G, D, E = c["heads"], c["kv_heads"], c["dim"], c["vdim"]
     f = rates(c["rot"]["base"], c["rot"]["dims"])
     q = rotate((h @ w[p + "q"].T).view(T, H, D), f, "pairs")
-    k = rotate((h @ w[p + "k"].T).view(T, G, D), f, "pairs")
-    v = (h @ w[p + "v"].T).view(T, G, E)
+    if kv is None:
+        k = rotate((h @ w[p + "k"].T).view(T, G, D), f, "pairs")
+        v = (h @ w[p + "v"].T).view(T, G, E)
+    else:
+        k, v = kv
     mask = chunk_mask(T, c["mask"]["size"]) if c.get("mask") else window_mask(T, None)
     o = attend(q, k, v, c["scale"], mask, w[p + "sink"])
     return o.reshape(T, H * E) @ w[p + "o"].T, (k, v)
@@ -217,10 +220,10 @@ class PlainNilepel:
         for i, layer in enumerate(c["layers"]):
             p, m = f"l{i}.", layer["mixer"]
             h = rms_norm(x, w[p + "norm1"], eps)
+            src = m.get("kv_from")
             if layer["type"] == "attention":
-                d, kept[i] = attention_chunked(h, w, p + "mix.", m)
+                d, kept[i] = attention_chunked(h, w, p + "mix.", m, None if src is None else kept[src])
             elif layer["type"] == "attention_2":
-                src = m.get("kv_from")
                 d, kept[i] = attention_windowed(h, w, p + "mix.", m, eps, None if src is None else kept[src])
             elif layer["type"] == "latent_attention":
                 d = latent_attention(h, w, p + "mix.", m, eps)

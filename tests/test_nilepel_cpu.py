@@ -31,10 +31,9 @@ def test_configuration_to_a_dict_and_back():
     (("layers", 0, "mixer", "kv_heads"), 3, "kv heads"),
     (("layers", 0, "mixer", "rot", "dims"), 7, "dims"),
     (("layers", 0, "mixer", "rot", "scaling", "high"), 0.5, "low < high"),
-    (("layers", 2, "mixer", "rot", "scaling"), {"factor": 2.0, "low": 1.0, "high": 2.0, "original": 8}, "scaling"),
     (("layers", 1, "mixer", "rot", "dims"), 10, "dims"),
     (("layers", 3, "mixer", "kv_from"), 3, "earlier layer"),
-    (("layers", 3, "mixer", "kv_from"), 2, "another type"),
+    (("layers", 3, "mixer", "kv_from"), 1, "another kind"),
     (("layers", 3, "mixer", "heads"), 2, "other head sizes"),
     (("layers", 1, "mlp", "router", "top"), 4, "top"),
     (("layers", 1, "mlp", "router", "groups", "count"), 4, "groups"),

@@ -277,10 +277,11 @@ def test_experts_with_a_factor_and_a_shared_expert_behind_its_gate(dtype):
 # ----------------------------------------------------------------------------- whole models
 
 def lengths(name):
-    return {"P": [1, 2, 21, 64, 65, 150], "Q": [3, 70, 71, 129, 140], "R": [5, 64, 128, 200], "S": [1, 2, 3, 66, 90]}[name]
+    return {"P": [1, 2, 21, 64, 65, 150], "Q": [3, 70, 71, 129, 140], "R": [5, 64, 128, 200], "S": [1, 2, 3, 66, 90],
+            "T": [2, 41, 100, 130]}[name]
 
 
-@pytest.mark.parametrize("name,dtype", cases(["P", "Q", "R", "S"]))
+@pytest.mark.parametrize("name,dtype", cases(["P", "Q", "R", "S", "T"]))
 def test_whole_prompts(name, dtype):
     eng = engine(name, dtype)
     for i, n in enumerate(lengths(name)):
@@ -332,7 +333,7 @@ def test_portions_of_several_sizes(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,head,n", [("P", 30, 130), ("Q", 1, 160), ("R", 100, 290), ("S", 3, 90)])
+@pytest.mark.parametrize("name,head,n", [("P", 30, 130), ("Q", 1, 160), ("R", 100, 290), ("S", 3, 90), ("T", 35, 100)])
 def test_prompt_then_token_by_token(name, head, n, dtype):
     """Decoding long enough that every window and run passes over decoded tokens and over a page's border."""
     if dtype not in [d for _, d in cases([name])]:
@@ -349,7 +350,7 @@ def test_prompt_then_token_by_token(name, head, n, dtype):
     eng.cache.check()
 
 
-@pytest.mark.parametrize("name,dtype", cases(["P", "Q", "R", "S"]))
+@pytest.mark.parametrize("name,dtype", cases(["P", "Q", "R", "S", "T"]))
 def test_unequal_batches_and_slots_used_again(name, dtype):
     """Requests of unequal lengths start together and are decoded together, the shorter ones ending earlier; then
     other requests take the slots and pages that came free (the cache has room for little more than one batch), in

@@ -24,13 +24,13 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import KvNeed
-from .linear import Matrix, linear, linear_for_sum
+from .linear import Matrix, linear, linear_for_sum, deferred_product
 from .mixer import Mixer, _projection
 from .position import Position, NoPosition
 
 
 class LatentAttention(Mixer):
-    takes_scaled_rows = False
+    takes_scaled_rows = True      # (as GatedWindowAttention: the products at both ends take a norm's halves)
     capturable = True
 
     NAMES = {"q": "q", "down": "dkv", "down_norm": "dkv.norm", "up_k": "uk", "up_v": "uv", "g": "g", "o": "o"}
@@ -118,4 +118,4 @@ class LatentAttention(Mixer):
         gate = proj[:, nh * (dim + rot) + R:] if self.gate else None
         ops.heads_product(o_lat.view(N, nh, rank), self.w_uv, o.view(N, nh, vdim), gate=gate,
                           gate_per_value=self.gate == "value")
-        return linear_for_sum(o, self.w_o)
+        return deferred_product(o, self.w_o)

@@ -217,7 +217,9 @@ class GatedWindowAttention(Mixer):
     Tensor names: prefix + "q", "k", "v", "o" (+ ".b" for their biases), "q.norm", "k.norm", "g", "sink"; `names`
     renames them.
     """
-    takes_scaled_rows = False
+    # (the input projection over packed weights finishes a norm's rows itself, and the output product without a bias
+    # is left for the following norm to run with the residual sum as its epilogue: parts.linear)
+    takes_scaled_rows = True
     capturable = True
 
     NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "g": "g", "q_norm": "q.norm", "k_norm": "k.norm", "bias": ".b",
@@ -349,8 +351,9 @@ class GatedWindowAttention(Mixer):
             # 32-bit, single tokens, and head sizes that the tiles do not take: a wave (or eight) for each (token, head)
             ops.window_attention(q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o, self.scale, self.nh,
                                  self.nkv, self.dim, self.vdim, **how)
-        y = linear_for_sum(o, self.w_o)
-        return WeightedDeltas([(y, 1.0, self.b_o)]) if self.b_o is not None else y
+        if self.b_o is None:
+            return deferred_product(o, self.w_o)
+        return WeightedDeltas([(linear_for_sum(o, self.w_o), 1.0, self.b_o)])
 
 
 class DifferentialAttention(Mixer):

@@ -1,4 +1,4 @@
-"""synaptix_amd: a small decoder library (Qwen3 dense, Bizipel, Kamivik, Repolix) with generation of its own for one MI355X."""
+"""synaptix_amd: a small decoder library (Qwen3 dense, Bizipel, Kamivik, Repolix, Nilepel) with generation of its own for one MI355X."""
 from .config import ConfigError, Qwen3Config, BizipelConfig, load_config, register_architecture, known_architectures
 from .weights import WeightError, write_random_model
 from .cache import CacheFull, CacheError

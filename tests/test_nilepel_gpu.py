@@ -162,7 +162,19 @@ def test_one_far_key_among_hundreds_and_the_first_keys_of_a_run(dtype):
         out = torch.empty((1, H * E), dtype=dtype, device=DEV)
         ops.window_attention(dev(qq[at].reshape(1, H * D), dtype), kp, vp, ints(order).view(1, 11), st.tok_seq, st.tok_pos, out,
                              1.0, H, G, D, E, window=window or 0, chunk=chunk or 0, sinks=torch.zeros(H, device=DEV))
-        assert float((out.cpu().double() - want).abs().max()) < (2e-4 if dtype == torch.float32 else 4e-2), (far, at, window, chunk)
+        tol = 2e-4 if dtype == torch.float32 else 4e-2
+        assert float((out.cpu().double() - want).abs().max()) < tol, (far, at, window, chunk)
+        # the same query among all queries of a prompt (in bf16 also in tiles on the matrix cores)
+        st = Step([(0, 0, at + 1)])
+        qd = dev(qq[:at + 1].reshape(at + 1, H * D), dtype)
+        how = dict(window=window or 0, chunk=chunk or 0, sinks=torch.zeros(H, device=DEV))
+        out = torch.empty((at + 1, H * E), dtype=dtype, device=DEV)
+        ops.window_attention(qd, kp, vp, ints(order).view(1, 11), st.tok_seq, st.tok_pos, out, 1.0, H, G, D, E, **how)
+        assert float((out[at:].cpu().double() - want).abs().max()) < tol, ("prompt", far, at, window, chunk)
+        if dtype == torch.bfloat16:
+            out = torch.empty((at + 1, H * E), dtype=dtype, device=DEV)
+            ops.window_attention_prefill_bf16(qd, kp, vp, ints(order).view(1, 11), st.seq_start, st.seq_past, out, 1.0, H, G, D, E, **how)
+            assert float((out[at:].cpu().double() - want).abs().max()) < tol, ("prompt in tiles", far, at, window, chunk)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

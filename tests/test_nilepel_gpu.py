@@ -395,6 +395,44 @@ def test_unequal_batches_and_slots_used_again(name, dtype):
     assert eng.cache.free_slots == 3
 
 
+@pytest.mark.parametrize("seed", list(range(7000, 7016)))
+def test_configurations_drawn_from_a_seed_in_float32(seed):
+    """Layer kinds, orders, head counts, sizes, masks, readers of other layers' keys and routers drawn from a seed (the
+    cases above are chosen; these are not): a prompt whole, then requests of unequal lengths cut at unequal places
+    and decoded together, 3 to 20 of them, against the plain model for each alone."""
+    import random
+    from nilepel_cases import random_model
+    from synaptix_amd import Engine
+    cfg, folder, plain = random_model(seed)
+    rng = random.Random(seed + 1)
+    g = torch.Generator().manual_seed(seed)
+    T = rng.choice([70, 150, 330])
+    lens = [T, 9, T // 2] + [rng.randint(2, T) for _ in range(rng.choice([0, 6, 10, 17]))]
+    toks = [torch.randint(0, cfg.vocab, (n,), generator=g).tolist() for n in lens]
+    want = [plain.logits(t) for t in toks]
+    eng = Engine.load(folder, dtype="float32", max_tokens=8192, max_slots=32)
+    s = eng.acquire()
+    assert_logits_close(eng.step([(s, toks[0])], want="all"), want[0], "float32", f"seed {seed} whole", sharp=True)
+    eng.release(s)
+    slots = [eng.acquire() for _ in toks]
+    cut = [min(max(1, len(t) - 12 - 3 * (i % 5)), len(t)) for i, t in enumerate(toks)]
+    out = eng.step([(s, t[:k]) for s, t, k in zip(slots, toks, cut)], want="all")
+    got, at = [[] for _ in toks], 0
+    for i, k in enumerate(cut):
+        got[i].append(out[at:at + k])
+        at += k
+    fed, live = list(cut), [i for i in range(len(toks)) if cut[i] < len(toks[i])]
+    while live:
+        out = eng.step([(slots[i], [toks[i][fed[i]]]) for i in live], want="last")
+        for j, i in enumerate(live):
+            got[i].append(out[j:j + 1])
+            fed[i] += 1
+        live = [i for i in live if fed[i] < len(toks[i])]
+    for i in range(len(toks)):
+        assert_logits_close(torch.cat(got[i]), want[i], "float32", f"seed {seed} request {i} of {len(toks)}", sharp=True)
+    eng.cache.check()
+
+
 def test_a_window_gives_its_pages_back():
     """A long sequence in a cache that holds far fewer tokens than it has: the groups that keep a window or a run give
     the pages behind it back as the sequence grows (the configuration has no layer that sees every key)."""
